@@ -1,6 +1,7 @@
 from .llama import ConfigError, LlamaConfig, RopeScaling
+from .tuvodra import TuvodraConfig
 from .registry import architectures, config_from_dict, load_config, register_architecture
 from .spec import ExtraPart, LayerSpec, ModelSpec, PartSpec, RunSpec
 
-__all__ = ["ConfigError", "LlamaConfig", "RopeScaling", "architectures", "config_from_dict",
+__all__ = ["ConfigError", "LlamaConfig", "TuvodraConfig", "RopeScaling", "architectures", "config_from_dict",
            "load_config", "register_architecture", "ExtraPart", "LayerSpec", "ModelSpec", "PartSpec", "RunSpec"]

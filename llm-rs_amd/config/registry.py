@@ -8,6 +8,7 @@ import os
 from typing import Any, Callable, Dict
 
 from .llama import ConfigError, LlamaConfig
+from .tuvodra import TuvodraConfig
 
 # name -> function(config dict) -> typed config with .model_spec() and .to_dict()
 _ARCHITECTURES: Dict[str, Callable[[Dict[str, Any]], Any]] = {}
@@ -23,6 +24,8 @@ def architectures():
 
 def config_from_dict(d: Dict[str, Any]):
     archs = d.get("architectures")
+    if not archs and isinstance(d.get("architecture"), str):     # files that name one architecture, in the singular
+        archs = [d["architecture"]]
     if not archs:
         raise ConfigError("missing config key: architectures")
     name = archs[0]
@@ -44,3 +47,4 @@ def load_config(path: str):
 
 
 register_architecture("LlamaForCausalLM", LlamaConfig.from_dict)
+register_architecture("Tuvodra", TuvodraConfig.from_dict)

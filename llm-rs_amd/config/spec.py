@@ -61,10 +61,16 @@ class ModelSpec:
     embedding_scale: float = 1.0    # the token table's rows are multiplied by this on their way into the stream
     logit_scale: float = 1.0        # logits are multiplied by this, and then,
     logit_softcap: float = 0.0      # if > 0, bent into (-cap, cap): cap * tanh(logit / cap)
+    # The residual stream kept as this many copies, all equal to the embedding at the start and summed before the
+    # final norm; what each block reads from them and writes back is the block arrangement's business (every block
+    # of such a model must be one that `takes_streams`).
+    streams: int = 1
 
     def validate(self) -> None:
         if not self.layers:
             raise ValueError("a model needs at least one layer")
+        if not 1 <= self.streams <= 16:
+            raise ValueError(f"the residual stream has 1 to 16 copies, not {self.streams}")
         for i, layer in enumerate(self.layers):
             names = [e.name for e in layer.extra]
             for e in layer.extra:

@@ -8,7 +8,14 @@ struct AttnArgs {
     int q_stride, out_stride;  // elements between tokens
     int window;                // 0: all keys up to the query's position
     float scale;
+    int v_dim;                 // width of a value (the cache's values and `out` have it); head_dim where keys and values are alike
+    // A penalty that grows with the logarithm of the distance, taken off the scaled score of query i and key j:
+    // dist_r1[head] * ln(1 + dist_r2[head] * (i - j)), in 32-bit.  Both null: none.
+    const float* dist_r1;
+    const float* dist_r2;
 };
+// Whether a call is the plain one (values as wide as keys, no distance penalty) that every kernel file takes.
+static inline bool attn_is_plain(const AttnArgs& a) { return a.v_dim == a.head_dim && a.dist_r1 == nullptr; }
 
 #if defined(__HIPCC__)
 // A step's entries bring their tokens as tiles of `per` tokens that never cross an entry; entries with one token

@@ -224,6 +224,7 @@ int llmrs_attention_f32_mfma(hipStream_t stream, const float* q, float* out, con
                              const int* block_table, const int* positions, const int* q_starts, int n_entries,
                              int skip_single, const AttnArgs& a) {
     int G = a.n_heads / a.n_kv_heads;
+    if (!attn_is_plain(a)) return 0;
     if (a.head_dim % 32 || a.head_dim > 256 || a.page_size % 4 || G > 32 || q_starts == nullptr) return 0;
     if (a.q_stride % 4 || a.out_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)out & 15) || ((uintptr_t)k_cache & 15) ||
         ((uintptr_t)v_cache & 15))
@@ -252,6 +253,7 @@ int llmrs_attention_f32_mfma_split(hipStream_t stream, const float* q, float* pa
                                    const int* block_table, const int* q_starts, const int* seq_lens, int n_entries,
                                    int max_chunks, const AttnArgs& a) {
     int G = a.n_heads / a.n_kv_heads;
+    if (!attn_is_plain(a)) return 0;
     if (a.head_dim % 32 || a.head_dim > 256 || a.page_size % 4 || G > 32 || q_starts == nullptr || seq_lens == nullptr) return 0;
     if (a.q_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) || ((uintptr_t)v_cache & 15) || ((uintptr_t)partial & 7))
         return 0;

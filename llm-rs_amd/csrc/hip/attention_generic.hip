@@ -27,9 +27,12 @@
 // elements at a load; the sums are the same either way.
 template <class T, bool VEC>
 __device__ __forceinline__ void walk_keys(const float* qs, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
-                                          const int* __restrict__ table, const AttnArgs& a, int kvh, int begin, int end,
-                                          float& m, float& l, float (&acc)[MAX_HEAD_DIM / 64]) {
-    int lane = threadIdx.x, hd = a.head_dim, ps = a.page_size;
+                                          const int* __restrict__ table, const AttnArgs& a, int kvh, int h, int pos,
+                                          int begin, int end, float& m, float& l, float (&acc)[MAX_HEAD_DIM / 64]) {
+    int lane = threadIdx.x, hd = a.head_dim, vd = a.v_dim, ps = a.page_size;
+    // the distance penalty of this head (query at `pos`): r1 ln(1 + r2 (pos - j)), or none
+    const bool far = a.dist_r1 != nullptr;
+    const float r1 = far ? a.dist_r1[h] : 0.0f, r2 = far ? a.dist_r2[h] : 0.0f;
     for (int t0 = begin; t0 < end; t0 += 64) {
         int j = t0 + lane;
         bool valid = j < end;
@@ -52,6 +55,7 @@ __device__ __forceinline__ void walk_keys(const float* qs, const T* __restrict__
                 for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], to_f32(kp[d]), dot);
             }
             s = dot * a.scale;
+            if (far) s -= r1 * logf(fmaf(r2, (float)(pos - j), 1.0f));
         }
         float m_new = fmaxf(m, wave_max(s));
         float p = valid ? expf(s - m_new) : 0.0f;
@@ -67,8 +71,8 @@ __device__ __forceinline__ void walk_keys(const float* qs, const T* __restrict__
 #pragma unroll
             for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) {
                 int d = lane + 64 * i;
-                if (d < hd)
-                    acc[i] = fmaf(pj, to_f32(v_cache[v_cache_index(pagej, kvh, offj, d, a.n_kv_heads, ps, hd)]), acc[i]);
+                if (d < vd)
+                    acc[i] = fmaf(pj, to_f32(v_cache[v_cache_index(pagej, kvh, offj, d, a.n_kv_heads, ps, vd)]), acc[i]);
             }
         }
     }
@@ -95,12 +99,12 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
     float m = -INFINITY, l = 0.0f;
     float acc[MAX_HEAD_DIM / 64] = {};
-    walk_keys<T, VEC>(qs, k_cache, v_cache, table, a, kvh, lo, pos + 1, m, l, acc);
-    T* orow = out + (size_t)t * a.out_stride + (size_t)h * hd;
+    walk_keys<T, VEC>(qs, k_cache, v_cache, table, a, kvh, h, pos, lo, pos + 1, m, l, acc);
+    T* orow = out + (size_t)t * a.out_stride + (size_t)h * a.v_dim;
 #pragma unroll
     for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) {
         int d = lane + 64 * i;
-        if (d < hd) orow[d] = from_f32<T>(acc[i] / l);
+        if (d < a.v_dim) orow[d] = from_f32<T>(acc[i] / l);
     }
 }
 
@@ -128,13 +132,13 @@ __global__ __launch_bounds__(64) void attention_generic_split_kernel(
     __syncthreads();
     float m = -INFINITY, l = 0.0f;
     float acc[MAX_HEAD_DIM / 64] = {};
-    walk_keys<T, VEC>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, begin, end, m, l, acc);
-    float* pp = partial + ((size_t)(e * a.n_heads + h) * max_chunks + ch) * (hd + 2);
+    walk_keys<T, VEC>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, h, pos, begin, end, m, l, acc);
+    float* pp = partial + ((size_t)(e * a.n_heads + h) * max_chunks + ch) * (a.v_dim + 2);
     if (lane == 0) { pp[0] = m; pp[1] = l; }
 #pragma unroll
     for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) {
         int d = lane + 64 * i;
-        if (d < hd) pp[2 + d] = acc[i];
+        if (d < a.v_dim) pp[2 + d] = acc[i];
     }
 }
 
@@ -144,10 +148,17 @@ __global__ __launch_bounds__(64) void attention_generic_split_kernel(
 #define GROUP_MAX_HEAD_DIM 256
 template <class T, bool VEC, int G>
 __device__ __forceinline__ void walk_keys_group(const float* qs, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
-                                                const int* __restrict__ table, const AttnArgs& a, int kvh, int begin, int end,
+                                                const int* __restrict__ table, const AttnArgs& a, int kvh, int pos, int begin, int end,
                                                 float (&m)[G], float (&l)[G], float (&acc)[G][GROUP_MAX_HEAD_DIM / 64]) {
     constexpr int NACC = GROUP_MAX_HEAD_DIM / 64;
-    int lane = threadIdx.x, hd = a.head_dim, ps = a.page_size;
+    int lane = threadIdx.x, hd = a.head_dim, vd = a.v_dim, ps = a.page_size;
+    const bool far = a.dist_r1 != nullptr;       // the heads' distance penalties, see walk_keys
+    float r1[G], r2[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        r1[g] = far ? a.dist_r1[kvh * G + g] : 0.0f;
+        r2[g] = far ? a.dist_r2[kvh * G + g] : 0.0f;
+    }
     for (int t0 = begin; t0 < end; t0 += 64) {
         int j = t0 + lane;
         bool valid = j < end;
@@ -180,7 +191,10 @@ __device__ __forceinline__ void walk_keys_group(const float* qs, const T* __rest
                 }
             }
 #pragma unroll
-            for (int g = 0; g < G; ++g) s[g] = dot[g] * a.scale;
+            for (int g = 0; g < G; ++g) {
+                s[g] = dot[g] * a.scale;
+                if (far) s[g] -= r1[g] * logf(fmaf(r2[g], (float)(pos - j), 1.0f));
+            }
         }
         float p[G];
 #pragma unroll
@@ -202,8 +216,8 @@ __device__ __forceinline__ void walk_keys_group(const float* qs, const T* __rest
 #pragma unroll
             for (int i = 0; i < NACC; ++i) {
                 int d = lane + 64 * i;
-                if (d < hd) {
-                    float v = to_f32(v_cache[v_cache_index(pagej, kvh, offj, d, a.n_kv_heads, ps, hd)]);
+                if (d < vd) {
+                    float v = to_f32(v_cache[v_cache_index(pagej, kvh, offj, d, a.n_kv_heads, ps, vd)]);
 #pragma unroll
                     for (int g = 0; g < G; ++g) acc[g][i] = fmaf(pj[g], v, acc[g][i]);
                 }
@@ -235,14 +249,14 @@ __global__ __launch_bounds__(64) void attention_generic_group_tokens_kernel(
 #pragma unroll
         for (int i = 0; i < NACC; ++i) acc[g][i] = 0.0f;
     }
-    walk_keys_group<T, VEC, G>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, lo, pos + 1, m, l, acc);
+    walk_keys_group<T, VEC, G>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, pos, lo, pos + 1, m, l, acc);
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        T* orow = out + (size_t)t * a.out_stride + (size_t)(kvh * G + g) * hd;
+        T* orow = out + (size_t)t * a.out_stride + (size_t)(kvh * G + g) * a.v_dim;
 #pragma unroll
         for (int i = 0; i < NACC; ++i) {
             int d = lane + 64 * i;
-            if (d < hd) orow[d] = from_f32<T>(acc[g][i] / l[g]);
+            if (d < a.v_dim) orow[d] = from_f32<T>(acc[g][i] / l[g]);
         }
     }
 }
@@ -274,15 +288,15 @@ __global__ __launch_bounds__(64) void attention_generic_group_kernel(
 #pragma unroll
         for (int i = 0; i < NACC; ++i) acc[g][i] = 0.0f;
     }
-    walk_keys_group<T, VEC, G>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, begin, end, m, l, acc);
+    walk_keys_group<T, VEC, G>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, pos, begin, end, m, l, acc);
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        float* pp = partial + ((size_t)(e * a.n_heads + kvh * G + g) * max_chunks + ch) * (hd + 2);
+        float* pp = partial + ((size_t)(e * a.n_heads + kvh * G + g) * max_chunks + ch) * (a.v_dim + 2);
         if (lane == 0) { pp[0] = m[g]; pp[1] = l[g]; }
 #pragma unroll
         for (int i = 0; i < NACC; ++i) {
             int d = lane + 64 * i;
-            if (d < hd) pp[2 + d] = acc[g][i];
+            if (d < a.v_dim) pp[2 + d] = acc[g][i];
         }
     }
 }
@@ -293,7 +307,7 @@ template <class T>
 __global__ __launch_bounds__(64) void attention_generic_merge_kernel(
     const float* __restrict__ partial, T* __restrict__ out, const int* __restrict__ q_starts,
     const int* __restrict__ seq_lens, int max_chunks, AttnArgs a) {
-    int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, hd = a.head_dim;
+    int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, hd = a.v_dim;     // (the rows added up are values)
     int t = q_starts[e];
     if (q_starts[e + 1] - t != 1) return;
     int pos = seq_lens[e] - 1;
@@ -363,12 +377,12 @@ static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cac
     bool vec = a.head_dim % 4 == 0 && (uintptr_t)k_cache % (4 * sizeof(T)) == 0;
     // Single-token entries are split by key range when the caller gave room for the partial results.
     int max_chunks = max_seq_len > 0 ? ceil_div(max_seq_len, GENERIC_CHUNK) : 0;
-    size_t need = (size_t)n_entries * a.n_heads * max_chunks * (a.head_dim + 2) * sizeof(float);
+    size_t need = (size_t)n_entries * a.n_heads * max_chunks * (a.v_dim + 2) * sizeof(float);
     bool split = max_chunks > 0 && scratch != nullptr && q_starts != nullptr && seq_lens != nullptr &&
                  scratch_bytes >= need && n_single != 0 && n_entries <= 65535 && max_chunks <= 65535;
     bool only_single = split && n_single == n_entries && a.n_tokens == n_entries;     // every entry brings one token: the caller says so
     const int G = a.n_heads / a.n_kv_heads;
-    const bool groupable = a.head_dim <= GROUP_MAX_HEAD_DIM && (G == 2 || G == 4 || G == 8);
+    const bool groupable = a.head_dim <= GROUP_MAX_HEAD_DIM && a.v_dim <= GROUP_MAX_HEAD_DIM && (G == 2 || G == 4 || G == 8);
     bool tiles_took = false;
     if constexpr (std::is_same<T, float>::value) {
         // 32-bit: entries with several tokens go to the matrix cores where the shape allows
@@ -447,25 +461,30 @@ static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cac
 // caller's word that every entry brings exactly one token (then token t is entry t, and q_starts is not read);
 // single_keys: how many keys those entries see together (windows counted), if the host knows (0: it does not):
 // the matrix-core kernels choose the keys per wave by it.
-extern "C" int llmrs_attention(hipStream_t stream, int dtype, const void* q, int q_stride, void* out, int out_stride,
-                               const void* k_cache, const void* v_cache, const int* block_table, int table_width,
-                               const int* token_entry, const int* positions, const int* q_starts,
-                               const int* seq_lens, int n_entries, int n_tokens, int n_heads, int n_kv_heads,
-                               int head_dim, int page_size, int num_pages, int window, float scale,
-                               void* scratch, size_t scratch_bytes, int max_seq_len, int n_single, long single_keys,
-                               int allow_mfma) {
-    LLMRS_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0, "attention: bad sizes");
+// v_dim: the width of a value (the cache's values are [page][kv_head][v_dim][slot], `out` has v_dim per head);
+// dist_r1, dist_r2: [n_heads] 32-bit, the logarithmic distance penalty of AttnArgs, or both null.
+extern "C" int llmrs_attention_ext(hipStream_t stream, int dtype, const void* q, int q_stride, void* out, int out_stride,
+                                   const void* k_cache, const void* v_cache, const int* block_table, int table_width,
+                                   const int* token_entry, const int* positions, const int* q_starts,
+                                   const int* seq_lens, int n_entries, int n_tokens, int n_heads, int n_kv_heads,
+                                   int head_dim, int page_size, int num_pages, int window, float scale,
+                                   void* scratch, size_t scratch_bytes, int max_seq_len, int n_single, long single_keys,
+                                   int allow_mfma, int v_dim, const float* dist_r1, const float* dist_r2) {
+    LLMRS_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && v_dim > 0, "attention: bad sizes");
+    LLMRS_REQUIRE(v_dim <= MAX_HEAD_DIM, "attention: value width %d exceeds %d", v_dim, MAX_HEAD_DIM);
+    LLMRS_REQUIRE((dist_r1 == nullptr) == (dist_r2 == nullptr), "attention: the distance penalty needs both of its tables");
     LLMRS_REQUIRE(n_heads % n_kv_heads == 0, "attention: %d heads are no multiple of %d kv heads", n_heads, n_kv_heads);
     LLMRS_REQUIRE(head_dim <= MAX_HEAD_DIM, "attention: head_dim %d exceeds %d", head_dim, MAX_HEAD_DIM);
     LLMRS_REQUIRE(page_size > 0 && table_width > 0 && num_pages > 0, "attention: bad cache geometry");
-    LLMRS_REQUIRE(q_stride >= n_heads * head_dim && out_stride >= n_heads * head_dim, "attention: row stride too short");
+    LLMRS_REQUIRE(q_stride >= n_heads * head_dim && out_stride >= n_heads * v_dim, "attention: row stride too short");
     LLMRS_REQUIRE(window >= 0, "attention: negative window");
     LLMRS_REQUIRE(n_heads <= 65535, "attention: too many heads for one launch");
     LLMRS_REQUIRE(n_single <= n_entries, "attention: %d single-token entries among %d entries", n_single, n_entries);
     LLMRS_REQUIRE(n_single != n_entries || n_tokens == n_entries,
                   "attention: every entry is said to bring one token, but %d entries bring %d tokens", n_entries, n_tokens);
     if (n_tokens == 0) return 0;
-    AttnArgs a{n_tokens, n_heads, n_kv_heads, head_dim, page_size, table_width, num_pages, q_stride, out_stride, window, scale};
+    AttnArgs a{n_tokens, n_heads, n_kv_heads, head_dim, page_size, table_width, num_pages, q_stride, out_stride, window, scale,
+               v_dim, dist_r1, dist_r2};
     if (dtype == LLMRS_BF16 && allow_mfma) {
         int took = llmrs_attention_bf16_mfma(stream, (const bf16*)q, (bf16*)out, (const bf16*)k_cache, (const bf16*)v_cache,
                                              block_table, token_entry, positions, q_starts, seq_lens, n_entries,
@@ -486,4 +505,17 @@ extern "C" int llmrs_attention(hipStream_t stream, int dtype, const void* q, int
     if (rc != 0) return -1;
     LLMRS_LAUNCH_CHECK("attention");
     return 0;
+}
+
+extern "C" int llmrs_attention(hipStream_t stream, int dtype, const void* q, int q_stride, void* out, int out_stride,
+                               const void* k_cache, const void* v_cache, const int* block_table, int table_width,
+                               const int* token_entry, const int* positions, const int* q_starts,
+                               const int* seq_lens, int n_entries, int n_tokens, int n_heads, int n_kv_heads,
+                               int head_dim, int page_size, int num_pages, int window, float scale,
+                               void* scratch, size_t scratch_bytes, int max_seq_len, int n_single, long single_keys,
+                               int allow_mfma) {
+    return llmrs_attention_ext(stream, dtype, q, q_stride, out, out_stride, k_cache, v_cache, block_table, table_width,
+                               token_entry, positions, q_starts, seq_lens, n_entries, n_tokens, n_heads, n_kv_heads,
+                               head_dim, page_size, num_pages, window, scale, scratch, scratch_bytes, max_seq_len, n_single,
+                               single_keys, allow_mfma, head_dim, nullptr, nullptr);
 }

@@ -1121,6 +1121,7 @@ int llmrs_attention_bf16_mfma(hipStream_t stream, const bf16* q, bf16* out, cons
                               size_t scratch_bytes, int max_seq_len, int n_single, long single_keys, const AttnArgs& a) {
     (void)token_entry;
     int G = a.n_heads / a.n_kv_heads;
+    if (!attn_is_plain(a)) return 0;
     if (a.page_size != 16 || a.head_dim % 32 || G > 32 || q_starts == nullptr) return 0;
     if (a.q_stride % 8 || a.out_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)out & 7)) return 0;
     if (n_entries > 65535 || a.n_kv_heads > 65535) return 0;

@@ -1,0 +1,88 @@
+// What lies between a q/k/v projection and attention for mixers that neither rotate nor leave q and k as they come:
+// biases, a norm of q and k to unit root mean square per head, and the write of k and v into the paged cache, in one
+// pass over the projection's 32-bit sums.
+//
+//   q[t, h, :] = unit(sums_q[t, h, :] + bias_q[h, :])      unit(x) = x / sqrt(mean(x^2) + eps) over the head (eps 0: x)
+//   k likewise, into its page; v[t, g, :] = sums_v + bias_v, into its page (values lie transposed, cache_layout.h).
+// Everything is computed in 32-bit and rounded once to the activation type on the way out.
+#include "cache_layout.h"
+#include "common.h"
+
+struct QkvFinishArgs {
+    int n_tokens, n_heads, n_kv_heads, head_dim, v_dim;
+    int in_stride, q_stride;       // elements between tokens in the sums and in q
+    int page_size, num_pages, write_kv;
+    float eps;                     // of the unit norm; 0: q and k are not normed
+};
+
+// One wave for each (token, head of q, k or v).
+template <class T>
+__global__ __launch_bounds__(64) void qkv_finish_kernel(const float* __restrict__ sums, const float* __restrict__ bias,
+                                                         T* __restrict__ q, const int* __restrict__ slot_map,
+                                                         T* __restrict__ k_cache, T* __restrict__ v_cache, QkvFinishArgs a) {
+    int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    bool is_q = head < a.n_heads, is_k = !is_q && head < a.n_heads + a.n_kv_heads;
+    if (!is_q && !a.write_kv) return;
+    int width = (is_q || is_k) ? a.head_dim : a.v_dim;
+    int col = is_q ? head * a.head_dim
+                   : is_k ? a.n_heads * a.head_dim + (head - a.n_heads) * a.head_dim
+                          : (a.n_heads + a.n_kv_heads) * a.head_dim + (head - a.n_heads - a.n_kv_heads) * a.v_dim;
+    const float* src = sums + (size_t)t * a.in_stride + col;
+    float x[8];            // features lane, lane + 64, ... (heads of up to 512)
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        int d = lane + 64 * i;
+        x[i] = d < width ? src[d] + (bias ? bias[col + d] : 0.0f) : 0.0f;
+        ss = fmaf(x[i], x[i], ss);
+    }
+    float inv = 1.0f;
+    if ((is_q || is_k) && a.eps > 0.0f) inv = 1.0f / sqrtf(wave_sum(ss) / (float)width + a.eps);
+    if (is_q) {
+        T* dst = q + (size_t)t * a.q_stride + col;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int d = lane + 64 * i;
+            if (d < width) dst[d] = from_f32<T>(x[i] * inv);
+        }
+        return;
+    }
+    int slot = slot_map[t];
+    if (slot < 0 || slot >= a.num_pages * a.page_size) return;  // never write outside the cache
+    int page = slot / a.page_size, off = slot % a.page_size;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        int d = lane + 64 * i;
+        if (d >= width) continue;
+        if (is_k)
+            k_cache[k_cache_index(page, head - a.n_heads, off, d, a.n_kv_heads, a.page_size, a.head_dim)] = from_f32<T>(x[i] * inv);
+        else
+            v_cache[v_cache_index(page, head - a.n_heads - a.n_kv_heads, off, d, a.n_kv_heads, a.page_size, a.v_dim)] = from_f32<T>(x[i]);
+    }
+}
+
+// sums: [n_tokens, in_stride] 32-bit, a token's q heads, then its k heads, then its v heads; bias: the same columns
+// (or null); q: [n_tokens, q_stride] in `dtype`; the caches in `dtype`; slot_map: [n_tokens] page * page_size + slot.
+// n_kv_heads 0: the projection has no k and v (a mixer that reads another's cache).
+extern "C" int llmrs_qkv_finish(hipStream_t stream, int dtype, const float* sums, int in_stride, const float* bias, void* q,
+                                int q_stride, const int* slot_map, void* k_cache, void* v_cache, int n_tokens, int n_heads,
+                                int n_kv_heads, int head_dim, int v_dim, int page_size, int num_pages, int write_kv, float eps) {
+    LLMRS_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0 && v_dim > 0, "qkv_finish: bad sizes");
+    LLMRS_REQUIRE(head_dim <= 512 && v_dim <= 512, "qkv_finish: heads of %d / %d features exceed 512", head_dim, v_dim);
+    LLMRS_REQUIRE(in_stride >= (n_heads + n_kv_heads) * head_dim + n_kv_heads * v_dim && q_stride >= n_heads * head_dim,
+                  "qkv_finish: row stride too short");
+    LLMRS_REQUIRE(eps >= 0.0f, "qkv_finish: negative eps");
+    LLMRS_REQUIRE(!write_kv || (page_size > 0 && num_pages > 0 && slot_map && k_cache && v_cache), "qkv_finish: no cache to write");
+    LLMRS_REQUIRE(n_heads + 2 * n_kv_heads <= 65535, "qkv_finish: too many heads for one launch");
+    if (n_tokens == 0) return 0;
+    QkvFinishArgs a{n_tokens, n_heads, n_kv_heads, head_dim, v_dim, in_stride, q_stride, page_size, num_pages, write_kv, eps};
+    dim3 grid(n_tokens, n_heads + 2 * n_kv_heads);
+    if (dtype == LLMRS_F32)
+        qkv_finish_kernel<float><<<grid, 64, 0, stream>>>(sums, bias, (float*)q, slot_map, (float*)k_cache, (float*)v_cache, a);
+    else if (dtype == LLMRS_BF16)
+        qkv_finish_kernel<bf16><<<grid, 64, 0, stream>>>(sums, bias, (bf16*)q, slot_map, (bf16*)k_cache, (bf16*)v_cache, a);
+    else
+        return llmrs_fail("qkv_finish: unknown dtype %d", dtype);
+    LLMRS_LAUNCH_CHECK("qkv_finish");
+    return 0;
+}

@@ -21,6 +21,13 @@ class Model:
             raise ValueError(f"the engine computes in float32 or bfloat16, not {dtype}")
         self.spec, self.dtype, self.device = spec, dtype, torch.device(device)
         self.blocks = [build_block(layer, dtype) for layer in spec.layers]
+        self.streams = int(spec.streams)
+        # (one copy handled by arrangements that take copies is still laid out as [1, T, hidden])
+        self.streamed = self.streams > 1 or any(block.takes_streams for block in self.blocks)
+        if self.streamed:
+            for i, block in enumerate(self.blocks):
+                if not block.takes_streams:
+                    raise ValueError(f"layer {i}: the arrangement {type(block).__name__} does not work on a stream kept in several copies")
         self.final_norm = build_norm(spec.final_norm, dtype) if spec.final_norm is not None else None
         self.embedding: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
@@ -106,8 +113,14 @@ class Model:
         [n_want, vocab] at the wanted rows, or None when none is wanted."""
         k = kernels()
         T = ctx.n_tokens
-        h = ctx.workspace("model.h", (T, self.spec.hidden_size), torch.float32)
-        k.embed_rows(h, self.embedding, ctx.tokens, self.spec.embedding_scale)
+        if self.streamed:
+            # [streams, T, hidden]: every copy starts as the embedding; blocks read and write all of them
+            h = ctx.workspace("model.h", (self.streams, T, self.spec.hidden_size), torch.float32)
+            k.embed_rows(h[0], self.embedding, ctx.tokens, self.spec.embedding_scale)
+            k.streams_copy_first(h)
+        else:
+            h = ctx.workspace("model.h", (T, self.spec.hidden_size), torch.float32)
+            k.embed_rows(h, self.embedding, ctx.tokens, self.spec.embedding_scale)
         ctx.note_left(h, None)
         for i, run in enumerate(self.spec.schedule):
             ctx.run_index = i
@@ -120,6 +133,8 @@ class Model:
             block.forward(ctx, h, cache_views[i])
             if not block.keeps_left_current:
                 ctx.note_left(h, None)
+            if ctx.after_run is not None:
+                ctx.after_run(i, h)
         ctx.norm_after_block = ctx.upcoming_norm = None
         if ctx.n_want == 0:
             return None
@@ -127,10 +142,14 @@ class Model:
         # rows and gathers after (src/arch/llama.rs:135-139), which is the same numbers.
         # (A step of few single tokens that wants them all: the last product has prepared the final norm, and the
         # output matrix's product finishes it; no norm kernel runs.)
-        x = self.final_norm.deferred(ctx, h) if ctx.wants_every_row and self.final_norm is not None else None
+        x = self.final_norm.deferred(ctx, h) if ctx.wants_every_row and self.final_norm is not None and not self.streamed else None
         if x is None:
             x = ctx.workspace("model.head_in", (ctx.n_want, self.spec.hidden_size), self.dtype)
-            if self.final_norm is not None:
+            if self.streamed:
+                # the stream is the sum of its copies: a norm that can reads them all at the wanted rows itself
+                if self.final_norm is None or not self.final_norm.forward_streams(ctx, h, None, x, ctx.want_rows):
+                    raise ValueError("a stream kept in several copies needs a final norm that reads them (forward_streams)")
+            elif self.final_norm is not None:
                 self.final_norm.forward(ctx, h, x, ctx.want_rows)
             else:       # no norm before the output matrix: the wanted rows of the stream, in the activation type
                 rows = x if self.dtype == torch.float32 else ctx.workspace("model.head_rows", x.shape, torch.float32)

@@ -82,6 +82,9 @@ class StepContext:
         self._left = None               # kernels.NextNorm that describes the stream as it stands, or None
         self._left_of = 0               # the stream it describes
         self._last_y = 0                # where the rows left last lie
+        # For whoever wants to look at the stream between layers (debugging, tests): called as after_run(run, h)
+        # after every run of the schedule.  None in service; a step with it set is never recorded.
+        self.after_run = None
 
     def workspace(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         return self._runner.workspace(name, shape, dtype)
@@ -341,7 +344,7 @@ class StepRunner:
         if self.time_device and self._pinned:
             self.started = torch.cuda.Event(enable_timing=True)
             self.started.record()
-        if graph_widths is None:
+        if graph_widths is None or ctx.after_run is not None:
             return self.model.forward(ctx, self.cache.views)
         # A decode step.  Everything the kernels take from the host must be the same for
         # every step of this key: sizes, addresses, and the bound on the context length.

@@ -21,7 +21,7 @@ TRACE_ROUND_TO = 64      # a request's tokens count towards --max-tokens rounded
 
 class TraceReplayer:
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16, device: str = "cuda",
-                 max_requests: int = 64):
+                 max_requests: int = 4):
         if TRACE_ROUND_TO % page_size:
             raise ValueError(f"page_size {page_size} must divide {TRACE_ROUND_TO}")
         num_pages = max(-(-max_tokens // page_size), 1)
@@ -72,8 +72,9 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time, each rounded up to a multiple of 64")
     ap.add_argument("--page-size", type=int, default=16)
+    ap.add_argument("--max-requests", type=int, default=4, help="requests that may be live at once: slots for per-request state")
     args = ap.parse_args(argv)
-    replayer = TraceReplayer(args.model, args.dtype, args.max_tokens, page_size=args.page_size)
+    replayer = TraceReplayer(args.model, args.dtype, args.max_tokens, page_size=args.page_size, max_requests=args.max_requests)
     return replay_lines(replayer, sys.stdin, args.out)
 
 

@@ -188,6 +188,14 @@ class HipKernels(Kernels):
             "llmrs_argmax_rows": [V, V, I, I, I, V, V, c_size_t],
             "llmrs_sample_rows": [V, V, I, I, I, V, V],
             "llmrs_place_ids": [V, V, I, V, V, V, I, I, I],
+            "llmrs_attention_ext": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, ctypes.c_long, I, I, V, V],
+            "llmrs_group_rmsnorm": [V, I, V, V, ctypes.c_long, I, V, V, V, I, I, I, F, V, V],
+            "llmrs_streams_mix": [V, V, ctypes.c_long, I, V, V, V, ctypes.c_long],
+            "llmrs_streams_copy_first": [V, V, ctypes.c_long, I, ctypes.c_long],
+            "llmrs_qkv_finish": [V, I, V, I, V, V, I, V, V, V, I, I, I, I, I, I, I, I, F],
+            "llmrs_mingru_scan": [V, I, V, I, V, V, V, ctypes.c_long, V, V, I, I, V, I],
+            "llmrs_causal_conv_silu": [V, I, V, I, V, V, V, ctypes.c_long, V, V, V, I, I, I, I, V, I],
+            "llmrs_selective_scan": [V, I, V, I, V, I, I, I, V, I, V, V, V, V, I, V, ctypes.c_long, V, V, V, I, I, I, V, I],
         }
         for name, args in sigs.items():
             fn = getattr(lib, name)
@@ -391,11 +399,18 @@ class HipKernels(Kernels):
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
                   n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1,
-                  single_keys=0) -> None:
-        """single_keys: how many keys the single-token entries see together (windows counted), 0 if unknown."""
+                  single_keys=0, value_dim=0, distance=None) -> None:
+        """single_keys: how many keys the single-token entries see together (windows counted), 0 if unknown.
+        value_dim: the width of a value where it is not a key's (0: the same).  distance: (r1, r2), float32 [n_heads]
+        each: r1[h] * ln(1 + r2[h] * (i - j)) is taken off the scaled score of query i and key j."""
         assert q.stride(1) == 1 and out.stride(1) == 1 and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype
         assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
-        assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim == v_cache.numel()
+        v_dim = int(value_dim) or head_dim
+        assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim and v_cache.numel() == num_pages * n_kv_heads * page_size * v_dim
+        if v_dim != head_dim or distance is not None:
+            return self._attention_ext(q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens, n_heads,
+                                       n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch, max_seq_len, n_single,
+                                       single_keys, v_dim, distance)
         T = q.shape[0]
         assert token_entry.shape[0] == T and positions.shape[0] == T and out.shape[0] == T
         moved = flops = 0
@@ -411,6 +426,123 @@ class HipKernels(Kernels):
                   block_table.shape[0], T, n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale,
                   _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size(), int(max_seq_len),
                   int(n_single), int(single_keys), int(self.allow_mfma))
+
+    def _attention_ext(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens, n_heads,
+                       n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch, max_seq_len, n_single, single_keys,
+                       v_dim, distance) -> None:
+        T = q.shape[0]
+        assert token_entry.shape[0] == T and positions.shape[0] == T and out.shape[0] == T
+        r1 = r2 = None
+        if distance is not None:
+            r1, r2 = distance
+            assert r1.dtype == r2.dtype == torch.float32 and r1.numel() == r2.numel() == n_heads and r1.is_contiguous() and r2.is_contiguous()
+        moved = flops = 0
+        if self.times is not None:
+            keys = int(seq_lens.sum().item())
+            seen = int((positions + 1).sum().item()) if window <= 0 else int((positions + 1).clamp(max=window).sum().item())
+            moved = (keys * n_kv_heads * (head_dim + v_dim) + T * n_heads * (head_dim + v_dim)) * q.element_size()
+            flops = 2 * seen * n_heads * (head_dim + v_dim)
+        self._run(f"attention {T} tokens" + (" (decode)" if n_single == block_table.shape[0] else ""), moved, flops, q.dtype,
+                  self.lib.llmrs_attention_ext,
+                  self._stream(), _code(q.dtype), _p(q), q.stride(0), _p(out), out.stride(0), _p(k_cache), _p(v_cache),
+                  _p(block_table), block_table.shape[1], _p(token_entry), _p(positions), _p(q_starts), _p(seq_lens),
+                  block_table.shape[0], T, n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale,
+                  _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size(), int(max_seq_len),
+                  int(n_single), int(single_keys), int(self.allow_mfma), v_dim, _p(r1), _p(r2))
+
+    # out[i, :] = weight * groupnorm(sum_s w_in[s] * x[s][rows[i] or i, :]); x: [T, D] or [S, T, D] float32
+    def group_rmsnorm(self, out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, groups: int,
+                      rows: Optional[torch.Tensor] = None, w_in: Optional[torch.Tensor] = None,
+                      zero: Optional[torch.Tensor] = None, combined: Optional[torch.Tensor] = None) -> None:
+        """The RMS norm in `groups` equal consecutive parts of the row.  `x` with three dimensions is several streams,
+        combined with the weights `w_in` (None: summed) before the norm.  `zero` [n, D] float32 is cleared on the way,
+        `combined` [n, D] float32 gets the combined rows."""
+        assert x.dtype == torch.float32 and weight.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous()
+        S = x.shape[0] if x.dim() == 3 else 1
+        D, n = x.shape[-1], out.shape[0]
+        assert out.shape[1] == D == weight.shape[0]
+        assert (rows is None and n == x.shape[-2]) or (rows is not None and rows.dtype == torch.int32 and rows.shape[0] == n)
+        assert w_in is None or (w_in.dtype == torch.float32 and w_in.numel() == S)
+        for extra in (zero, combined):
+            assert extra is None or (extra.dtype == torch.float32 and extra.is_contiguous() and tuple(extra.shape) == (n, D))
+        self._run(f"group_rmsnorm {n}x{D}" + (f" of {S} streams" if S > 1 else ""), n * D * (4 * S + out.element_size()) + D * 4,
+                  (2 * S + 5) * n * D, None, self.lib.llmrs_group_rmsnorm, self._stream(), _code(out.dtype), _p(out), _p(x),
+                  x.stride(0) if x.dim() == 3 else 0, S, _p(w_in), _p(weight), _p(rows), n, D, int(groups), float(eps),
+                  _p(zero), _p(combined))
+
+    # x[r] = sum_s mix[s, r] * x[s] + w_out[r] * y, all streams at once from the old ones; x: [S, T, D] float32
+    def streams_mix(self, x: torch.Tensor, mix: torch.Tensor, w_out: torch.Tensor, y: torch.Tensor) -> None:
+        assert x.dim() == 3 and x.dtype == y.dtype == mix.dtype == w_out.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous()
+        S = x.shape[0]
+        assert tuple(mix.shape) == (S, S) and mix.is_contiguous() and w_out.numel() == S and y.numel() == x[0].numel()
+        self._run(f"streams_mix {S}x{y.shape[0]}x{y.shape[1]}", (2 * S + 1) * y.numel() * 4, 2 * S * S * y.numel(), None,
+                  self.lib.llmrs_streams_mix, self._stream(), _p(x), x.stride(0), S, _p(mix), _p(w_out), _p(y), y.numel())
+
+    # x[s] = x[0] for every s
+    def streams_copy_first(self, x: torch.Tensor) -> None:
+        assert x.dim() == 3 and x.dtype == torch.float32 and x.is_contiguous()
+        self._run("streams_copy_first", (x.shape[0] + 1) * x[0].numel() * 4, 0, None,
+                  self.lib.llmrs_streams_copy_first, self._stream(), _p(x), x.stride(0), x.shape[0], x[0].numel())
+
+    def qkv_finish(self, sums: torch.Tensor, bias: Optional[torch.Tensor], q: torch.Tensor, slot_map, k_cache, v_cache,
+                   n_heads: int, n_kv_heads: int, head_dim: int, v_dim: int, page_size: int, num_pages: int, write_kv: bool,
+                   eps: float) -> None:
+        """sums [T, q | k | v] float32 -> q [T, heads * head_dim] (activation type) and the cache's pages: biases
+        added, q and k divided by their root mean square over the head (eps > 0), one rounding on the way out."""
+        assert sums.dtype == torch.float32 and sums.stride(1) == 1 and q.stride(1) == 1 and q.shape[0] == sums.shape[0]
+        width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * v_dim
+        assert sums.shape[1] == width and (bias is None or (bias.dtype == torch.float32 and bias.numel() == width and bias.is_contiguous()))
+        if write_kv:
+            assert k_cache.dtype == v_cache.dtype == q.dtype and k_cache.is_contiguous() and v_cache.is_contiguous()
+            assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim and v_cache.numel() == num_pages * n_kv_heads * page_size * v_dim
+            assert slot_map.dtype == torch.int32 and slot_map.shape[0] == sums.shape[0]
+        T = sums.shape[0]
+        self._run("qkv_finish", T * width * (4 + q.element_size()), 4 * T * width, None, self.lib.llmrs_qkv_finish,
+                  self._stream(), _code(q.dtype), _p(sums), sums.stride(0), _p(bias), _p(q), q.stride(0), _p(slot_map),
+                  _p(k_cache), _p(v_cache), T, n_heads, n_kv_heads, head_dim, v_dim, page_size, num_pages, int(write_kv), float(eps))
+
+    def mingru_scan(self, sums: torch.Tensor, bias_z, bias_c, state: torch.Tensor, q_starts, slots, width: int, out: torch.Tensor) -> None:
+        """sums [T, gate | candidate | output gate] float32; state [slots, width] float32, read and left; out [T, width]."""
+        assert sums.dtype == torch.float32 and sums.stride(1) == 1 and sums.shape[1] == 3 * width and out.stride(1) == 1
+        assert state.dtype == torch.float32 and state.stride(-1) == 1 and state.shape[1] >= width and out.shape == (sums.shape[0], width)
+        assert q_starts.dtype == slots.dtype == torch.int32 and q_starts.numel() == slots.numel() + 1
+        for b in (bias_z, bias_c):
+            assert b is None or (b.dtype == torch.float32 and b.numel() == width)
+        T = sums.shape[0]
+        self._run(f"mingru_scan {T}x{width}", T * width * (12 + out.element_size()), 12 * T * width, None, self.lib.llmrs_mingru_scan,
+                  self._stream(), _code(out.dtype), _p(sums), sums.stride(0), _p(bias_z), _p(bias_c), _p(state), state.stride(0),
+                  _p(q_starts), _p(slots), slots.numel(), width, _p(out), out.stride(0))
+
+    def causal_conv_silu(self, sums: torch.Tensor, taps: torch.Tensor, bias, state: torch.Tensor, q_starts, slots, token_entry,
+                         channels: int, out: torch.Tensor) -> None:
+        """out[t, c] = silu(bias[c] + sum_j taps[c, j] * x[t - (K - 1 - j), c]) over the first `channels` columns x of
+        sums (float32); state [slots, >= (K - 1) * channels] float32 holds each request's last K - 1 inputs and is brought up to date."""
+        K = taps.shape[1]
+        assert sums.dtype == taps.dtype == state.dtype == torch.float32 and sums.stride(1) == 1 and taps.is_contiguous() and taps.shape[0] == channels
+        assert state.stride(-1) == 1 and state.shape[1] >= (K - 1) * channels and out.shape == (sums.shape[0], channels) and out.stride(1) == 1
+        assert q_starts.dtype == slots.dtype == token_entry.dtype == torch.int32 and token_entry.numel() == sums.shape[0]
+        T = sums.shape[0]
+        self._run(f"causal_conv {T}x{channels}", T * channels * (4 + out.element_size()), 2 * K * T * channels, None,
+                  self.lib.llmrs_causal_conv_silu, self._stream(), _code(out.dtype), _p(sums), sums.stride(0), _p(taps), _p(bias),
+                  _p(state), state.stride(0), _p(q_starts), _p(slots), _p(token_entry), slots.numel(), T, channels, K, _p(out), out.stride(0))
+
+    def selective_scan(self, x: torch.Tensor, bc: torch.Tensor, off_b: int, off_c: int, dt: torch.Tensor, dt_bias, A: torch.Tensor,
+                       D: torch.Tensor, gate: torch.Tensor, state: torch.Tensor, q_starts, slots, out: torch.Tensor,
+                       ypart: Optional[torch.Tensor] = None) -> None:
+        """S[c, n] <- exp(step_c A[c, n]) S[c, n] + step_c x_c B_n, y_c = sum_n S[c, n] C_n + D_c x_c, out = y * silu(gate),
+        step = softplus(dt + dt_bias); x, bc (B at column off_b, C at off_c) and out in the activation type, dt and gate
+        float32 [T, channels], state [slots, >= channels * states] float32, read and left."""
+        C, N = A.shape
+        T = x.shape[0]
+        assert x.dtype == bc.dtype == out.dtype and x.stride(1) == bc.stride(1) == out.stride(1) == 1 and x.shape[1] == C
+        assert dt.dtype == gate.dtype == A.dtype == D.dtype == state.dtype == torch.float32 and A.is_contiguous() and D.numel() == C
+        assert dt.stride(1) == gate.stride(1) == 1 and dt.shape == (T, C) and gate.shape == (T, C) and out.shape == (T, C)
+        assert state.stride(-1) == 1 and state.shape[1] >= C * N and (dt_bias is None or (dt_bias.dtype == torch.float32 and dt_bias.numel() == C))
+        assert ypart is None or (ypart.dtype == torch.float32 and ypart.is_contiguous() and ypart.numel() >= T * C)
+        self._run(f"selective_scan {T}x{C}x{N}", T * (C * (8 + 2 * x.element_size()) + 2 * N * x.element_size()), 7 * T * C * N, None,
+                  self.lib.llmrs_selective_scan, self._stream(), _code(x.dtype), _p(x), x.stride(0), _p(bc), bc.stride(0), int(off_b),
+                  int(off_c), _p(dt), dt.stride(0), _p(dt_bias), _p(A), _p(D), _p(gate), gate.stride(0), _p(state), state.stride(0),
+                  _p(ypart), _p(q_starts), _p(slots), slots.numel(), C, N, _p(out), out.stride(0))
 
     def argmax_rows(self, logits: torch.Tensor, out: torch.Tensor, scratch: Optional[torch.Tensor] = None) -> None:
         """`scratch`: 256 bytes per row let several blocks share a long row."""

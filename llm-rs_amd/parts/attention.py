@@ -11,6 +11,12 @@ their pages by the same kernel (for a few tokens) or the next; attention of
 every query token over its request's pages; h += o Wo^T with the sum fused into
 the product.  No biases.
 
+Options for mixers that prepare q and k otherwise (all off for Llama): `value_dim` (values of another width than
+keys), `bias` (q, k and v have biases), `qk_norm_eps` (q and k are divided by their root mean square over the head,
+with this eps, no weight), `distance` = "log" (a per-head penalty r1 ln(1 + r2 (i - j)) taken off the scaled score,
+with the head's numbers in two tensors), `names` (the leaves of the tensors' names).  With any of them the q/k/v
+product leaves 32-bit sums, and one kernel adds the biases, norms q and k and writes k and v into their pages.
+
 The rotation kernels pair neighbours (2i, 2i+1).  Where the encoding pairs
 (i, i + rotary_dim/2), the rows of Wq and Wk are reordered within each head at
 load so that those two features become neighbours: q.k is a sum over features
@@ -24,7 +30,7 @@ import math
 import torch
 
 from ..cache.spec import PagedKV
-from ..kernels import EPI_ACCUM_F32, EPI_STORE, kernels
+from ..kernels import EPI_ACCUM_F32, EPI_STORE, EPI_STORE_F32, kernels
 from .base import Mixer, TensorSpec, build_position, place, register_mixer
 
 
@@ -50,15 +56,42 @@ class Attention(Mixer):
             raise ValueError(f"{self.heads} heads are no multiple of {self.kv_heads} kv heads")
         self.q_size = self.heads * self.head_dim
         self.kv_size = self.kv_heads * self.head_dim
+        self.value_dim = int(p.get("value_dim") or self.head_dim)
+        self.v_size = self.kv_heads * self.value_dim
+        self.o_size = self.heads * self.value_dim
+        self.has_bias = bool(p.get("bias", False))
+        self.qk_norm_eps = float(p.get("qk_norm_eps") or 0.0)
+        self.distance = p.get("distance")
+        if self.distance not in (None, "log"):
+            raise ValueError(f"unknown distance penalty {self.distance!r} (known: log)")
+        # q and k are prepared by a kernel of their own between the product and attention
+        self.prepared = self.has_bias or self.qk_norm_eps > 0 or self.distance is not None or self.value_dim != self.head_dim
+        if self.prepared and self.position is not None:
+            raise ValueError("a position encoding together with biases, a q/k norm, a distance penalty or values of another width is not built")
+        if self.prepared:
+            self.recording_signature = None
+        leaves = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+                  "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "r1": "r1", "r2": "r2",
+                  **(p.get("names") or {})}
+        self.names = {key: self.name(leaf) for key, leaf in leaves.items()}
         self.w_qkv = None
         self.w_o = None
+        self.bias = self.r1 = self.r2 = None
 
     def tensors(self):
-        t = {self.name("q_proj.weight"): TensorSpec((self.q_size, self.hidden)),
-             self.name("o_proj.weight"): TensorSpec((self.hidden, self.q_size))}
+        n = self.names
+        t = {n["q"]: TensorSpec((self.q_size, self.hidden)), n["o"]: TensorSpec((self.hidden, self.o_size))}
         if self.kv_proj:
-            t[self.name("k_proj.weight")] = TensorSpec((self.kv_size, self.hidden))
-            t[self.name("v_proj.weight")] = TensorSpec((self.kv_size, self.hidden))
+            t[n["k"]] = TensorSpec((self.kv_size, self.hidden))
+            t[n["v"]] = TensorSpec((self.v_size, self.hidden))
+        if self.has_bias:
+            t[n["q_bias"]] = TensorSpec((self.q_size,))
+            if self.kv_proj:
+                t[n["k_bias"]] = TensorSpec((self.kv_size,))
+                t[n["v_bias"]] = TensorSpec((self.v_size,))
+        if self.distance is not None:
+            t[n["r1"]] = TensorSpec((self.heads,), "normal:0.5:0.2")
+            t[n["r2"]] = TensorSpec((self.heads,), "normal:0.5:0.05")     # 1 + r2 (i - j) must stay positive
         return t
 
     def _pair_neighbours(self, w: torch.Tensor, heads: int, undo: bool = False) -> torch.Tensor:
@@ -74,29 +107,67 @@ class Attention(Mixer):
         return w.view(heads, self.head_dim, -1)[:, order.to(w.device), :].reshape(w.shape)
 
     def load(self, tensors, device):
-        get = lambda n: place(tensors[self.name(n)], device, self.dtype)
-        parts = [self._pair_neighbours(get("q_proj.weight"), self.heads)]
+        get = lambda n: place(tensors[self.names[n]], device, self.dtype)
+        get32 = lambda n: place(tensors[self.names[n]], device, torch.float32)
+        parts = [self._pair_neighbours(get("q"), self.heads)]
         if self.kv_proj:
-            parts += [self._pair_neighbours(get("k_proj.weight"), self.kv_heads), get("v_proj.weight")]
+            parts += [self._pair_neighbours(get("k"), self.kv_heads), get("v")]
         self.w_qkv = torch.cat(parts, dim=0).contiguous()
-        self.w_o = get("o_proj.weight")
+        self.w_o = get("o")
+        if self.has_bias:       # added to the 32-bit sums: kept in 32-bit, side by side as the product's columns are
+            self.bias = torch.cat([get32("q_bias")] + ([get32("k_bias"), get32("v_bias")] if self.kv_proj else [])).contiguous()
+        if self.distance is not None:
+            self.r1, self.r2 = get32("r1"), get32("r2")
         if self.position is not None:
             self.position.to(device)
 
     def export(self):
         w = self.w_qkv.cpu()
-        out = {self.name("q_proj.weight"): self._pair_neighbours(w[:self.q_size], self.heads, undo=True).contiguous(),
-               self.name("o_proj.weight"): self.w_o.cpu()}
+        n = self.names
+        out = {n["q"]: self._pair_neighbours(w[:self.q_size], self.heads, undo=True).contiguous(), n["o"]: self.w_o.cpu()}
         if self.kv_proj:
             k, v = w[self.q_size:self.q_size + self.kv_size], w[self.q_size + self.kv_size:]
-            out[self.name("k_proj.weight")] = self._pair_neighbours(k, self.kv_heads, undo=True).contiguous()
-            out[self.name("v_proj.weight")] = v.contiguous()
+            out[n["k"]] = self._pair_neighbours(k, self.kv_heads, undo=True).contiguous()
+            out[n["v"]] = v.contiguous()
+        if self.has_bias:
+            b = self.bias.cpu()
+            out[n["q_bias"]] = b[:self.q_size].contiguous()
+            if self.kv_proj:
+                out[n["k_bias"]] = b[self.q_size:self.q_size + self.kv_size].contiguous()
+                out[n["v_bias"]] = b[self.q_size + self.kv_size:].contiguous()
+        if self.distance is not None:
+            out[n["r1"]], out[n["r2"]] = self.r1.cpu(), self.r2.cpu()
         return out
 
     def cache_need(self):
-        return PagedKV(self.kv_heads, self.head_dim, self.window)
+        return PagedKV(self.kv_heads, self.head_dim, self.window, self.value_dim if self.value_dim != self.head_dim else 0)
+
+    def _forward_prepared(self, ctx, x, h, cache):
+        """The product's 32-bit sums -> biases, unit norm of q and k, cache write -> attention with the distance penalty."""
+        k = kernels()
+        T = x.shape[0]
+        write = self.kv_proj and cache.writes
+        n_kv = self.kv_heads if self.kv_proj else 0
+        g = cache.group
+        sums = ctx.workspace("attn.sums", (T, self.w_qkv.shape[0]), torch.float32)
+        k.gemm(x, self.w_qkv, sums, EPI_STORE_F32, ctx.gemm_workspace(x, self.w_qkv))
+        q = ctx.workspace("attn.qkv", (T, self.q_size), self.dtype)
+        k.qkv_finish(sums, self.bias, q, ctx.slot_maps[g], cache.k, cache.v, self.heads, n_kv, self.head_dim, self.value_dim,
+                     cache.page_size, cache.num_pages, write, self.qk_norm_eps)
+        o = ctx.workspace("attn.out", (T, self.o_size), self.dtype)
+        need = k.attention_scratch_floats(ctx.n_entries, self.heads, max(self.head_dim, self.value_dim), ctx.max_seq_len,
+                                          self.kv_heads, ctx.n_single) if ctx.n_single else 0
+        scratch = ctx.workspace("attn.partial", (need,), torch.float32) if need else None
+        k.attention(q, o, cache.k, cache.v, ctx.block_tables[g], ctx.token_entry, ctx.positions, ctx.q_starts, ctx.seq_lens,
+                    self.heads, self.kv_heads, self.head_dim, cache.page_size, cache.num_pages, self.window, self.scale,
+                    scratch, ctx.max_seq_len, ctx.n_single, 0, value_dim=self.value_dim,
+                    distance=None if self.distance is None else (self.r1, self.r2))
+        k.gemm(o, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(o, self.w_o))
+        ctx.note_left(h, None)
 
     def takes_normed_rows(self, ctx, rows):
+        if self.prepared:
+            return False
         # the q/k/v product norms its rows itself where it is the fused kernel: a rotation it applies (or none)
         fused = self.position is None or self.position.rotary() is not None
         return fused and kernels().product_norms_its_rows(rows, self.w_qkv.shape[0], self.hidden, self.dtype)
@@ -110,7 +181,7 @@ class Attention(Mixer):
 
     def recording_key(self, ctx):
         k = kernels()
-        if not ctx.n_single:
+        if not ctx.n_single or self.prepared:
             return 0
         keys = ctx.single_keys(self.window)
         want = k.attention_split_chunk(ctx.n_single, self.kv_heads, self.head_dim, ctx.max_seq_len, keys)
@@ -133,6 +204,8 @@ class Attention(Mixer):
         return ctx.single_keys(self.window)
 
     def forward(self, ctx, x, h, cache):
+        if self.prepared:
+            return self._forward_prepared(ctx, x, h, cache)
         k = kernels()
         T = x.shape[0]
         write = self.kv_proj and cache.writes

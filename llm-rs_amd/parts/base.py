@@ -110,6 +110,12 @@ class Norm(Part):
         (`kernels.NextNorm` with eps); None for any other norm."""
         return None
 
+    def forward_streams(self, ctx, hs: torch.Tensor, w_in: Optional[torch.Tensor], out: torch.Tensor,
+                        rows: Optional[torch.Tensor] = None, zero: Optional[torch.Tensor] = None) -> bool:
+        """out[i] = norm(sum_s w_in[s] * hs[s][rows[i]]) for a stream kept as copies hs [S, T, D] (w_in None: the plain
+        sum; zero: [n, D] float32 to clear on the way).  False: this norm cannot read several copies."""
+        return False
+
     def deferred(self, ctx, h: torch.Tensor):
         """The norm of every row of `h`, not computed here: a `kernels.NormedRows` for a part that
         `takes_normed_rows`, or the normed rows themselves (a tensor) where the last product that added into `h`
@@ -162,6 +168,8 @@ class Block:
     # `forward`, and what an earlier product left was dropped before that part ran).  The model drops
     # it after any block that does not say so.
     keeps_left_current = False
+    # True for an arrangement whose `forward` takes the stream as several copies, h [streams, T, hidden].
+    takes_streams = False
 
     def first_norm(self) -> Optional[Norm]:
         """The norm that reads the stream first when this block runs, if the block before may prepare it."""

@@ -9,7 +9,12 @@ from .base import Block, register_block
 
 
 class PreNormBlock(Block):
-    needs = ("mixer", "feed_forward", "mixer_norm", "feed_forward_norm")
+    def __init__(self, named):
+        super().__init__(named)
+        if self.feed_forward is not None and self.feed_forward_norm is None:
+            raise ValueError("block arrangement PreNormBlock needs the parts feed_forward_norm")
+
+    needs = ("mixer", "mixer_norm")      # a layer may have no feed-forward; one that has needs its norm too
     keeps_left_current = True       # `normed_input` drops what was left before each part; the feed-forward runs last
 
     def first_norm(self):
@@ -17,6 +22,10 @@ class PreNormBlock(Block):
 
     def forward(self, ctx, h, cache):
         after = ctx.norm_after_block
+        if self.feed_forward is None:
+            self.mixer.forward(ctx, self.normed_input(ctx, h, self.mixer_norm, self.mixer, after), h, cache)
+            ctx.upcoming_norm = None
+            return
         self.mixer.forward(ctx, self.normed_input(ctx, h, self.mixer_norm, self.mixer, self.feed_forward_norm), h, cache)
         self.feed_forward.forward(ctx, self.normed_input(ctx, h, self.feed_forward_norm, self.feed_forward, after), h)
         ctx.upcoming_norm = None

@@ -19,24 +19,27 @@ class SwiGLU(FeedForward):
         super().__init__(spec, dtype)
         self.hidden = int(spec.params["hidden_size"])
         self.inter = int(spec.params["intermediate_size"])
+        # the leaves of the three tensors' names, for files that call them otherwise: {"gate": ..., "up": ..., "down": ...}
+        leaves = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight", **(spec.params.get("names") or {})}
+        self.n_gate, self.n_up, self.n_down = (self.name(leaves[k]) for k in ("gate", "up", "down"))
         self.w_gate_up = None
         self.w_down = None
 
     def tensors(self):
-        return {self.name("gate_proj.weight"): TensorSpec((self.inter, self.hidden)),
-                self.name("up_proj.weight"): TensorSpec((self.inter, self.hidden)),
-                self.name("down_proj.weight"): TensorSpec((self.hidden, self.inter))}
+        return {self.n_gate: TensorSpec((self.inter, self.hidden)),
+                self.n_up: TensorSpec((self.inter, self.hidden)),
+                self.n_down: TensorSpec((self.hidden, self.inter))}
 
     def load(self, tensors, device):
-        gate = place(tensors[self.name("gate_proj.weight")], device, self.dtype)
-        up = place(tensors[self.name("up_proj.weight")], device, self.dtype)
+        gate = place(tensors[self.n_gate], device, self.dtype)
+        up = place(tensors[self.n_up], device, self.dtype)
         self.w_gate_up = torch.stack([gate, up], dim=1).reshape(2 * self.inter, self.hidden).contiguous()
-        self.w_down = place(tensors[self.name("down_proj.weight")], device, self.dtype)
+        self.w_down = place(tensors[self.n_down], device, self.dtype)
 
     def export(self):
         both = self.w_gate_up.cpu().view(self.inter, 2, self.hidden)
-        return {self.name("gate_proj.weight"): both[:, 0, :].contiguous(), self.name("up_proj.weight"): both[:, 1, :].contiguous(),
-                self.name("down_proj.weight"): self.w_down.cpu()}
+        return {self.n_gate: both[:, 0, :].contiguous(), self.n_up: both[:, 1, :].contiguous(),
+                self.n_down: self.w_down.cpu()}
 
     def takes_normed_rows(self, ctx, rows):
         return kernels().product_norms_its_rows(rows, 2 * self.inter, self.hidden, self.dtype)

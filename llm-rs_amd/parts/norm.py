@@ -48,3 +48,41 @@ class RMSNorm(Norm):
 
 
 register_norm("rmsnorm", RMSNorm)
+
+
+class GroupRMSNorm(Norm):
+    """RMS norm in groups(size, eps, groups): the row is cut into `groups` equal consecutive parts, each part p becomes
+    p / sqrt(mean(p^2) + eps), and the whole is multiplied by the weight; 32-bit throughout.  groups = 1 is RMSNorm.
+    It also reads a stream kept in several copies, combined with given weights on the way (`forward_streams`).
+    `tensor`: the leaf of the weight's name ("weight"); "" when the prefix itself is the name."""
+    graph_safe = True
+
+    def __init__(self, spec, dtype):
+        super().__init__(spec, dtype)
+        self.size = int(spec.params["size"])
+        self.eps = float(spec.params["eps"])
+        self.groups = int(spec.params.get("groups", 1))
+        if self.groups < 1 or self.size % self.groups:
+            raise ValueError(f"a row of {self.size} does not fall into {self.groups} equal groups")
+        leaf = spec.params.get("tensor", "weight")
+        self.weight_name = self.name(leaf) if leaf else self.prefix
+        self.weight = None
+
+    def tensors(self):
+        return {self.weight_name: TensorSpec((self.size,), "norm")}
+
+    def load(self, tensors, device):
+        self.weight = place(tensors[self.weight_name], device, torch.float32)
+
+    def export(self):
+        return {self.weight_name: self.weight.cpu()}
+
+    def forward(self, ctx, h, out, rows=None):
+        kernels().group_rmsnorm(out, h, self.weight, self.eps, self.groups, rows)
+
+    def forward_streams(self, ctx, hs, w_in, out, rows=None, zero=None):
+        kernels().group_rmsnorm(out, hs, self.weight, self.eps, self.groups, rows, w_in=w_in, zero=zero)
+        return True
+
+
+register_norm("group_rmsnorm", GroupRMSNorm)

@@ -24,14 +24,24 @@ def _tensor_seed(seed: int, name: str) -> int:
     return int.from_bytes(h[:8], "little") & (2**63 - 1)
 
 
+def normal_of_kind(kind: str) -> Tuple[float, float]:
+    """(mean, standard deviation) that a part asks for its tensor in random-weights mode (`TensorSpec.kind`)."""
+    if kind == "norm":
+        return 1.0, 0.1
+    if kind.startswith("normal:"):
+        _, mean, std = kind.split(":")
+        return float(mean), float(std)
+    return 0.0, 0.02
+
+
 def random_tensors(shapes: Mapping[str, Tuple[int, ...]], kinds: Mapping[str, str], seed: int,
                    dtype=torch.bfloat16, device="cpu") -> Dict[str, torch.Tensor]:
-    """`kinds[name]` is "matrix" (N(0, 0.02)) or "norm" (1 + N(0, 0.1))."""
+    """`kinds[name]` is "matrix" (N(0, 0.02)), "norm" (1 + N(0, 0.1)) or "normal:<mean>:<std>"."""
     if dtype not in (torch.float32, torch.bfloat16):
         raise ValueError(f"random weights are made in float32 or bfloat16, not {dtype}")
     out = {}
     for name, shape in shapes.items():
-        mean, std = (1.0, 0.1) if kinds[name] == "norm" else (0.0, 0.02)
+        mean, std = normal_of_kind(kinds[name])
         out[name] = fill_normal(torch.empty(tuple(shape), dtype=dtype, device=device), _tensor_seed(seed, name), mean, std)
     return out
 
