@@ -16,9 +16,19 @@ logarithmic distance penalty; an optional gated feed-forward; logits through the
 from __future__ import annotations
 
 import math
-from typing import Dict, List, Optional, Sequence
+from typing import Callable, Dict, List, Optional, Sequence
 
 import torch
+
+# `rnd` in the functions below: applied to every activation that one stage hands the next through memory in an
+# implementation that keeps such hand-overs in 16 bits (never to the streams, to a state, or to anything the design
+# wants in 32-bit).  The identity by default; the tests pass a rounding to bfloat16 to learn how far rounding alone
+# takes a model from its exact logits.
+_same = lambda x: x
+
+
+def bf16_rounding(x: torch.Tensor) -> torch.Tensor:
+    return x.to(torch.bfloat16).to(x.dtype)
 
 
 def plain_group_rmsnorm(x: torch.Tensor, w: Optional[torch.Tensor], eps: float, groups: int) -> torch.Tensor:
@@ -43,7 +53,7 @@ def plain_softplus(x: torch.Tensor) -> torch.Tensor:
     return torch.where(x > 30.0, x, torch.log1p(torch.exp(torch.clamp(x, max=30.0))))
 
 
-def plain_mingru(h: torch.Tensor, w: Dict[str, torch.Tensor]) -> torch.Tensor:
+def plain_mingru(h: torch.Tensor, w: Dict[str, torch.Tensor], rnd: Callable = _same) -> torch.Tensor:
     """h: [T, D].  gate z_t = sigmoid(Wz h_t + bz); u_t = Wx h_t + bx; candidate c_t = u_t + 1/2 where u_t >= 0,
     sigmoid(u_t) elsewhere; s_t = (1 - z_t) s_{t-1} + z_t c_t from s = 0; out_t = Wo (s_t * silu(Wg h_t))."""
     z = plain_sigmoid(h @ w["z"].T + w["z.b"])
@@ -55,7 +65,7 @@ def plain_mingru(h: torch.Tensor, w: Dict[str, torch.Tensor]) -> torch.Tensor:
     for t in range(h.shape[0]):
         s = (1.0 - z[t]) * s + z[t] * cand[t]
         rows.append(s * gate[t])
-    return torch.stack(rows) @ w["o"].T
+    return rnd(torch.stack(rows)) @ w["o"].T
 
 
 def plain_causal_conv(x: torch.Tensor, taps: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
@@ -74,15 +84,15 @@ def plain_causal_conv(x: torch.Tensor, taps: torch.Tensor, bias: torch.Tensor) -
     return y
 
 
-def plain_mamba1(h: torch.Tensor, w: Dict[str, torch.Tensor], dt_rank: int, n_state: int) -> torch.Tensor:
+def plain_mamba1(h: torch.Tensor, w: Dict[str, torch.Tensor], dt_rank: int, n_state: int, rnd: Callable = _same) -> torch.Tensor:
     """Selective scan.  [x | g] = Win h; x <- silu(conv(x)); [d | B | C] = Wx x; step = softplus(Wdt d + bdt) per
     channel; A = -exp(A_log); S[c, n] <- exp(step_c A[c, n]) S[c, n] + step_c x_c B_n; y_c = sum_n S[c, n] C_n +
     D_c x_c; out = Wo (y * silu(g))."""
     inner = w["in"].shape[0] // 2
     xg = h @ w["in"].T
     x, g = xg[:, :inner], xg[:, inner:]
-    x = plain_silu(plain_causal_conv(x, w["conv"], w["conv.b"]))
-    p = x @ w["x"].T
+    x = rnd(plain_silu(plain_causal_conv(x, w["conv"], w["conv.b"])))
+    p = rnd(x @ w["x"].T)
     d, B, C = p[:, :dt_rank], p[:, dt_rank:dt_rank + n_state], p[:, dt_rank + n_state:dt_rank + 2 * n_state]
     step = plain_softplus(d @ w["dt"].T + w["dt.b"])
     A = -torch.exp(w["A_log"])
@@ -91,12 +101,12 @@ def plain_mamba1(h: torch.Tensor, w: Dict[str, torch.Tensor], dt_rank: int, n_st
     for t in range(h.shape[0]):
         S = torch.exp(step[t][:, None] * A) * S + (step[t] * x[t])[:, None] * B[t][None, :]
         rows.append(S @ C[t] + w["D"] * x[t])
-    y = torch.stack(rows) * plain_silu(g)
+    y = rnd(torch.stack(rows) * plain_silu(g))
     return y @ w["o"].T
 
 
 def plain_window_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], heads: int, kv_heads: int, dim: int, vdim: int,
-                           scale: float, window: int, eps: float) -> torch.Tensor:
+                           scale: float, window: int, eps: float, rnd: Callable = _same) -> torch.Tensor:
     """q, k, v with biases; q and k divided by their root mean square over `dim`, head by head; score(i, j) =
     q_i . k_j * scale - r1_h ln(1 + r2_h (i - j)) for 0 <= i - j < window; softmax over those j; heads side by side
     through Wo.  Query head a reads key/value head a // (heads / kv_heads)."""
@@ -104,8 +114,9 @@ def plain_window_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], heads: i
     q = (h @ w["q"].T + w["q.b"]).reshape(T, heads, dim)
     k = (h @ w["k"].T + w["k.b"]).reshape(T, kv_heads, dim)
     v = (h @ w["v"].T + w["v.b"]).reshape(T, kv_heads, vdim)
-    q = plain_group_rmsnorm(q, None, eps, 1)
-    k = plain_group_rmsnorm(k, None, eps, 1)
+    q = rnd(plain_group_rmsnorm(q, None, eps, 1))
+    k = rnd(plain_group_rmsnorm(k, None, eps, 1))
+    v = rnd(v)
     per = heads // kv_heads
     out = torch.zeros(T, heads, vdim, dtype=h.dtype)
     for a in range(heads):
@@ -116,11 +127,11 @@ def plain_window_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], heads: i
             s = (k[lo:i + 1, g] @ q[i, a]) * scale - w["r1"][a] * torch.log(1.0 + w["r2"][a] * dist)
             p = torch.softmax(s, dim=0)
             out[i, a] = p @ v[lo:i + 1, g]
-    return out.reshape(T, heads * vdim) @ w["o"].T
+    return rnd(out.reshape(T, heads * vdim)) @ w["o"].T
 
 
-def plain_gated_mlp(h: torch.Tensor, w: Dict[str, torch.Tensor]) -> torch.Tensor:
-    return (plain_silu(h @ w["gate"].T) * (h @ w["up"].T)) @ w["down"].T
+def plain_gated_mlp(h: torch.Tensor, w: Dict[str, torch.Tensor], rnd: Callable = _same) -> torch.Tensor:
+    return rnd(plain_silu(h @ w["gate"].T) * (h @ w["up"].T)) @ w["down"].T
 
 
 def plain_hyper_step(xs: torch.Tensor, hc: Dict[str, torch.Tensor], sublayer) -> torch.Tensor:
@@ -137,7 +148,7 @@ def _sub(tensors, prefix, compute):
 
 
 def plain_tuvodra_logits(cfg: dict, tensors: Dict[str, torch.Tensor], tokens: Sequence[int], compute=torch.float64,
-                         layers_out: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
+                         layers_out: Optional[List[torch.Tensor]] = None, rnd: Callable = _same) -> torch.Tensor:
     """Logits [T, vocab] of one sequence.  `layers_out`, if a list, gets the sum of the streams after each layer."""
     eps, groups, S = float(cfg["norm"]["eps"]), int(cfg["norm"]["groups"]), int(cfg["streams"])
     table = tensors["embed"].to(compute)
@@ -148,21 +159,21 @@ def plain_tuvodra_logits(cfg: dict, tensors: Dict[str, torch.Tensor], tokens: Se
         m, kind = layer["mixer"], layer["type"]
         mw = _sub(tensors, f"{p}.mix", compute)
         if kind == "mingru":
-            mixer = lambda h: plain_mingru(h, mw)
+            mixer = lambda h: plain_mingru(h, mw, rnd)
         elif kind == "mamba1":
-            mixer = lambda h: plain_mamba1(h, mw, int(m["dt_rank"]), int(m["state"]))
+            mixer = lambda h: plain_mamba1(h, mw, int(m["dt_rank"]), int(m["state"]), rnd)
         elif kind == "attention":
             mixer = lambda h: plain_window_attention(h, mw, int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"]),
-                                                     float(m["scale"]), int(m["mask"]["size"]), eps)
+                                                     float(m["scale"]), int(m["mask"]["size"]), eps, rnd)
         else:
             raise ValueError(kind)
         n1 = tensors[f"{p}.norm1"].to(compute)
-        xs = plain_hyper_step(xs, _sub(tensors, f"{p}.hc1", compute), lambda u: mixer(plain_group_rmsnorm(u, n1, eps, groups)))
+        xs = plain_hyper_step(xs, _sub(tensors, f"{p}.hc1", compute), lambda u: mixer(rnd(plain_group_rmsnorm(u, n1, eps, groups))))
         if layer.get("mlp") is not None:
             n2 = tensors[f"{p}.norm2"].to(compute)
             fw = _sub(tensors, f"{p}.mlp", compute)
-            xs = plain_hyper_step(xs, _sub(tensors, f"{p}.hc2", compute), lambda u: plain_gated_mlp(plain_group_rmsnorm(u, n2, eps, groups), fw))
+            xs = plain_hyper_step(xs, _sub(tensors, f"{p}.hc2", compute), lambda u: plain_gated_mlp(rnd(plain_group_rmsnorm(u, n2, eps, groups)), fw, rnd))
         if layers_out is not None:
             layers_out.append(xs.sum(dim=0))
-    x = plain_group_rmsnorm(xs.sum(dim=0), tensors["final.norm"].to(compute), eps, groups)
+    x = rnd(plain_group_rmsnorm(xs.sum(dim=0), tensors["final.norm"].to(compute), eps, groups))
     return x @ table.T
