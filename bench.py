@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b|prompts|long|widths|portions]
+    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b|prompts|long|widths|portions|tuvodra]
 
 The default run (`decode8b`) is the Llama-3.1-8B shape with random bfloat16 weights: 8
 requests, each with 2,048 tokens of context in the cache, decode K steps through the
@@ -63,7 +63,7 @@ LLAMA_8B = _llama(32, 4096, 32, 8, 128, 14336, 8.0, False)
 LLAMA_1B = _llama(16, 2048, 32, 8, 64, 8192, 32.0, True)
 LLAMA_70B = _llama(80, 8192, 64, 8, 128, 28672, 8.0, False)
 SHAPES = {"Llama-3.1-8B shape": LLAMA_8B, "Llama-3.2-1B shape": LLAMA_1B, "Llama-3.1-70B shape": LLAMA_70B}
-WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts", "long", "widths", "portions")
+WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts", "long", "widths", "portions", "tuvodra")
 
 
 def flat_config(model: str, layers_run: int, global_batch: int, seq_len: int, page_size: int, **more) -> dict:
@@ -198,12 +198,12 @@ def prompts_line(args, layers, points, fractions, first_step_s=0.0) -> dict:
 class Bench:
     def __init__(self, args, shape: dict, num_pages: int, max_requests: int, max_batch_tokens: int):
         import torch
-        from llm_rs_amd import Engine, LlamaConfig
+        from llm_rs_amd import Engine, config_from_dict
         self.torch = torch
         d = dict(shape)
-        if args.layers:
+        if args.layers and "num_hidden_layers" in d:
             d["num_hidden_layers"] = args.layers
-        self.config = LlamaConfig.from_dict(d)
+        self.config = config_from_dict(d)
         t0 = time.time()
         self.engine = Engine.from_random(self.config, seed=0, dtype=args.dtype, device="cuda:0", page_size=16,
                                          num_pages=num_pages, max_requests=max_requests, max_batch_tokens=max_batch_tokens)
@@ -213,7 +213,7 @@ class Bench:
         self.gen = torch.Generator().manual_seed(0)
 
     def prompt(self, n):
-        return self.torch.randint(0, self.config.vocab_size, (n,), generator=self.gen).tolist()
+        return self.torch.randint(0, self.engine.model.spec.vocab_size, (n,), generator=self.gen).tolist()
 
     def timed(self, fn, reps):
         self.torch.cuda.synchronize()
@@ -537,6 +537,71 @@ def run_portions(args) -> dict:
     return line
 
 
+# ---- the Tuvodra decoder beside the Llama decoder at equal widths ---------------------------------------------------
+
+def tuvodra_shape(width, heads, kv_heads, dim, ff, window, repeats, vocab=128256):
+    """Layers in threes: a minGRU as wide as the stream, a selective scan twice as wide with 16 states, and windowed
+    attention with a feed-forward, each of the sizes the Llama shape of that width has."""
+    three = [{"type": "mingru", "mixer": {"width": width}, "mlp": None},
+             {"type": "mamba1", "mixer": {"inner": 2 * width, "state": 16, "conv": 4, "dt_rank": width // 16}, "mlp": None},
+             {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                             "mask": {"size": window}}, "mlp": {"kind": "dense", "ff": ff}}]
+    return {"architecture": "Tuvodra", "vocab": vocab, "width": width, "streams": 4, "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-5, "groups": 2}, "layers": [dict(l) for _ in range(repeats) for l in three]}
+
+
+def run_tuvodra(args) -> dict:
+    """Prompt and decode throughput of the Tuvodra decoder at two widths, each beside a Llama decoder of the same
+    width, heads, feed-forward and number of layers (random weights both)."""
+    from llm_rs_amd import StepEntry
+    from llm_rs_amd.kernels import kernels
+    repeats = max(1, (args.layers or 6) // 3)
+    T, batch, context = args.prefill_tokens, args.batch, args.context
+    sizes = {"1B widths": (LLAMA_1B, 2048, 32, 8, 64, 8192), "8B widths": (LLAMA_8B, 4096, 32, 8, 128, 14336)}
+    points = {}
+    for size, (llama, width, heads, kv_heads, dim, ff) in sizes.items():
+        if args.only_size and args.only_size not in size:
+            continue
+        pair = {"tuvodra": tuvodra_shape(width, heads, kv_heads, dim, ff, args.window, repeats),
+                "llama": dict(llama, num_hidden_layers=3 * repeats)}
+        for name, shape in pair.items():
+            b = Bench(args, shape, batch * (context + 256) // 16 + T // 16 + 64, max(batch, 8), max(T, 2048))
+            engine = b.engine
+            toks = b.prompt(T)
+
+            def prompt_once():
+                slot = engine.open_request()
+                engine.step([StepEntry(slot, 0, toks, [T - 1])])
+                engine.close_request(slot)
+
+            prompt_once()
+            prefill_s = b.timed(prompt_once, max(2, min(args.steps // 8, 8)))
+            if kernels().times is not None:
+                print(f"[bench] {name}, {size}: kernels of a prompt of {T} tokens", file=sys.stderr)
+                kernels().times.dump()
+            step_s, _ = b.decode_run(batch, context, args.steps, args.warmup)
+            if kernels().times is not None:
+                print(f"[bench] {name}, {size}: kernels of decoding, {batch} requests over {context} tokens", file=sys.stderr)
+                kernels().times.dump()
+            weights = engine.model.weight_bytes_per_step()
+            points[f"{name} {size}"] = {"prefill_tokens_per_s": round(T / prefill_s, 1), "prefill_ms": round(prefill_s * 1e3, 3),
+                                        "decode_tokens_per_s": round(batch / step_s, 1), "decode_ms_per_step": round(step_s * 1e3, 4),
+                                        "weight_bytes_per_step": weights, "decode_frac_of_hbm_weights_only": round(weights / step_s / PEAK_HBM, 4)}
+            print(f"[bench] {name}, {size}: prompt of {T} tokens {prefill_s * 1e3:.2f} ms, decode step {step_s * 1e3:.3f} ms", file=sys.stderr, flush=True)
+            del b, engine
+            import gc
+            gc.collect()
+            import torch
+            torch.cuda.empty_cache()
+    first = next(iter(points.values()))
+    line = base_line("decode_tokens_per_s", first["decode_tokens_per_s"], args.steps, args.warmup, first["decode_ms_per_step"] * 1e-3, args.dtype,
+                     {"model": "Tuvodra (minGRU, selective scan, windowed attention + feed-forward, in threes) beside Llama of equal widths",
+                      "global_batch": batch, "seq_len": context, "parallelism": "single GPU", "layers_run": 3 * repeats,
+                      "prefill_tokens": T, "window": args.window, "streams": 4, "page_size": 16})
+    line["points"] = points
+    return line
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -554,6 +619,8 @@ def main() -> int:
     ap.add_argument("--requests", type=int, default=256, help="serve1b: requests submitted at once")
     ap.add_argument("--new-tokens", type=int, default=256, help="serve1b: tokens generated for each request")
     ap.add_argument("--max-batch-tokens", type=int, default=2048, help="serve1b: tokens a scheduler step may run")
+    ap.add_argument("--window", type=int, default=1024, help="tuvodra: keys an attention layer sees")
+    ap.add_argument("--only-size", default="", help="tuvodra: run one of the sizes only (1B or 8B)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -562,7 +629,7 @@ def main() -> int:
     args.steps = args.steps if args.steps is not None else (8 if heavy else 64)
     args.warmup = args.warmup if args.warmup is not None else (2 if heavy else 8)
     line = {"decode8b": run_decode8b, "serve1b": run_serve1b, "mixed70b": run_mixed70b, "sizes": run_sizes, "sizes1b": run_sizes,
-            "prompts": run_prompts, "long": run_long, "widths": run_widths, "portions": run_portions}[args.workload](args)
+            "prompts": run_prompts, "long": run_long, "widths": run_widths, "portions": run_portions, "tuvodra": run_tuvodra}[args.workload](args)
     from llm_rs_amd.kernels import kernels
     if kernels().times is not None:         # LLM_PERF: what was still to be shown of the per-kernel table
         kernels().times.dump()

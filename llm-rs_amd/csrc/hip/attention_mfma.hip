@@ -72,8 +72,20 @@ __device__ __forceinline__ float other_half(float x) {
 // for tiles that lie wholly inside every column's range.
 #define SOFTMAX_SLACK 8.0f
 #define ATTN_WIDE_FROM_KEYS 32768        // tiles of eight waves from this bound on the step's lengths
+// With `far` (the same in all lanes) a penalty that grows with the logarithm of the distance is taken off first:
+// S c - r1 log2(1 + r2 (pos - key)), which is (score - r1 ln(1 + r2 d)) log2(e); r1 and r2 are the column's head's.
 __device__ __forceinline__ bool softmax_tile(f32x16& S, float& m, float& l, int t0, int pos, int lo,
-                                             int h, float c, float& alpha, bool edge) {
+                                             int h, float c, float& alpha, bool edge,
+                                             bool far = false, float r1 = 0.0f, float r2 = 0.0f) {
+    if (far) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            int key = t0 + 16 * (i >> 3) + 8 * h + 4 * ((i >> 2) & 1) + (i & 3);
+            float d = (float)max(pos - key, 0);           // (keys past the query are masked below)
+            S[i] = __builtin_fmaf(S[i], c, -r1 * __builtin_amdgcn_logf(__builtin_fmaf(r2, d, 1.0f)));
+        }
+        c = 1.0f;
+    }
     if (edge) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
@@ -114,7 +126,8 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
                                              const bf16* __restrict__ kc, const bf16* __restrict__ vc,
                                              const int* __restrict__ table, int table_width, int num_pages,
                                              int n_kv, int kvh, int t_begin, int t_end, int pos, int lo, float scale,
-                                             bool have_pages = false, int first_pages = 0) {
+                                             bool have_pages = false, int first_pages = 0,
+                                             bool far = false, float r1 = 0.0f, float r2 = 0.0f) {
     int lane = threadIdx.x & 63;
     int r = lane & 31, h = lane >> 5;
     float scale_log2e = scale * 1.44269504088896341f;
@@ -184,7 +197,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
             vf[dt][0] = *(const bf16x8*)(vp0 + dt * 32 * 16);
             vf[dt][1] = *(const bf16x8*)(vp1 + dt * 32 * 16);
         }
-        bool moved = softmax_tile(S, m, l, t0, pos, lo, h, scale_log2e, alpha_out, __any(t0 + 31 > pos || t0 < lo));
+        bool moved = softmax_tile(S, m, l, t0, pos, lo, h, scale_log2e, alpha_out, __any(t0 + 31 > pos || t0 < lo), far, r1, r2);
         float alpha = alpha_out;
         bf16x8 pf[2];
 #pragma unroll
@@ -248,7 +261,8 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(const bf16* __restrict_
         for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
     float m = -INFINITY, l = 0.0f;
     attend_range<HD>(qf, O, m, l, kc, vc, block_table + (size_t)e * a.table_width, a.table_width, a.num_pages,
-                     a.n_kv_heads, kvh, t_begin, t_end, pos, lo, a.scale);
+                     a.n_kv_heads, kvh, t_begin, t_end, pos, lo, a.scale, false, 0,
+                     a.dist_r1 != nullptr, a.dist_r1 ? a.dist_r1[head] : 0.0f, a.dist_r1 ? a.dist_r2[head] : 0.0f);
     if (!cvalid) return;
     float inv = 1.0f / l;
     bf16* op = out + (size_t)token * a.out_stride + (size_t)head * HD;
@@ -344,6 +358,8 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(HD <
         for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
     float m = -INFINITY, l = 0.0f;
     float scale_log2e = a.scale * 1.44269504088896341f;
+    const bool far = a.dist_r1 != nullptr;                           // the distance penalty of this column's head
+    const float far_r1 = far ? a.dist_r1[head] : 0.0f, far_r2 = far ? a.dist_r2[head] : 0.0f;
 
     // ---- loads.  A tile's keys are two pages and so are its values; each wave brings its share of a
     // page of both (page wave & 1, share wave >> 1: half a page with four waves, a quarter with eight).  What a lane fetches for its place in the page's
@@ -489,11 +505,11 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(HD <
             if (is_edge(t)) {
                 S_next = scores((s + 1) % R);         // (nothing real for the last tile: not used then)
                 read_values(s, vf);
-                moved = softmax_tile(S_cur, m, l, t_begin + 32 * t, pos, lo, h, scale_log2e, alpha, true);
+                moved = softmax_tile(S_cur, m, l, t_begin + 32 * t, pos, lo, h, scale_log2e, alpha, true, far, far_r1, far_r2);
             } else {
                 S_next = scores((s + 1) % R);
                 read_values(s, vf);
-                moved = softmax_tile(S_cur, m, l, t_begin + 32 * t, pos, lo, h, scale_log2e, alpha, false);
+                moved = softmax_tile(S_cur, m, l, t_begin + 32 * t, pos, lo, h, scale_log2e, alpha, false, far, far_r1, far_r2);
             }
             to_bf16(S_cur, pf);
             rescale(moved, alpha);
@@ -570,7 +586,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 3
         for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
     float m = -INFINITY, l = 0.0f;
     attend_range<HD>(qf, O, m, l, kc, vc, table, a.table_width, a.num_pages,
-                     a.n_kv_heads, kvh, t_begin, t_end, pos, lo_t, a.scale, plain != 0, first_pages);
+                     a.n_kv_heads, kvh, t_begin, t_end, pos, lo_t, a.scale, plain != 0, first_pages,
+                     a.dist_r1 != nullptr, a.dist_r1 ? a.dist_r1[head] : 0.0f, a.dist_r1 ? a.dist_r2[head] : 0.0f);
     if (!cvalid) return;
     float* pp = partial + ((size_t)(e * a.n_heads + head) * max_chunks + ch) * (HD + 2);
     if (h == 0) { pp[0] = m; pp[1] = l; }
@@ -659,7 +676,10 @@ __global__ __launch_bounds__(64) void attn_split16_kernel(const bf16* __restrict
     }
     int t_end = min(t_begin + chunk, pos_t + 1);
     int pv_base = t_begin >> 4;
-    float c2 = a.scale * 1.44269504088896341f;
+    const bool far = a.dist_r1 != nullptr;
+    const float far_r1 = far ? a.dist_r1[head] : 0.0f, far_r2 = far ? a.dist_r2[head] : 0.0f;
+    const float c2s = a.scale * 1.44269504088896341f;
+    float c2 = far ? 1.0f : c2s;                      // with the penalty the scores are brought to base 2 before the maximum
     f32x4 O[HD / 16];
 #pragma unroll
     for (int dt = 0; dt < HD / 16; ++dt) O[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -719,6 +739,13 @@ __global__ __launch_bounds__(64) void attn_split16_kernel(const bf16* __restrict
         float sc[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) sc[i] = S[i >> 2][i & 3];
+        if (far) {                                                    // (the same in all lanes) the distance penalty, base 2
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float d = (float)max(pos_t - (t0 + 8 * g + i), 0);
+                sc[i] = __builtin_fmaf(sc[i], c2s, -far_r1 * __builtin_amdgcn_logf(__builtin_fmaf(far_r2, d, 1.0f)));
+            }
+        }
         if (t0 + 31 > pos_t || t0 < lo_t) {                           // (the same in all lanes)
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -1121,7 +1148,7 @@ int llmrs_attention_bf16_mfma(hipStream_t stream, const bf16* q, bf16* out, cons
                               size_t scratch_bytes, int max_seq_len, int n_single, long single_keys, const AttnArgs& a) {
     (void)token_entry;
     int G = a.n_heads / a.n_kv_heads;
-    if (!attn_is_plain(a)) return 0;
+    if (a.v_dim != a.head_dim) return 0;               // (a distance penalty is these kernels' too)
     if (a.page_size != 16 || a.head_dim % 32 || G > 32 || q_starts == nullptr) return 0;
     if (a.q_stride % 8 || a.out_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)out & 7)) return 0;
     if (n_entries > 65535 || a.n_kv_heads > 65535) return 0;

@@ -68,8 +68,6 @@ class Attention(Mixer):
         self.prepared = self.has_bias or self.qk_norm_eps > 0 or self.distance is not None or self.value_dim != self.head_dim
         if self.prepared and self.position is not None:
             raise ValueError("a position encoding together with biases, a q/k norm, a distance penalty or values of another width is not built")
-        if self.prepared:
-            self.recording_signature = None
         leaves = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
                   "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "r1": "r1", "r2": "r2",
                   **(p.get("names") or {})}
@@ -160,7 +158,7 @@ class Attention(Mixer):
         scratch = ctx.workspace("attn.partial", (need,), torch.float32) if need else None
         k.attention(q, o, cache.k, cache.v, ctx.block_tables[g], ctx.token_entry, ctx.positions, ctx.q_starts, ctx.seq_lens,
                     self.heads, self.kv_heads, self.head_dim, cache.page_size, cache.num_pages, self.window, self.scale,
-                    scratch, ctx.max_seq_len, ctx.n_single, 0, value_dim=self.value_dim,
+                    scratch, ctx.max_seq_len, ctx.n_single, self._keys_for_the_split(ctx), value_dim=self.value_dim,
                     distance=None if self.distance is None else (self.r1, self.r2))
         k.gemm(o, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(o, self.w_o))
         ctx.note_left(h, None)
@@ -181,7 +179,7 @@ class Attention(Mixer):
 
     def recording_key(self, ctx):
         k = kernels()
-        if not ctx.n_single or self.prepared:
+        if not ctx.n_single:
             return 0
         keys = ctx.single_keys(self.window)
         want = k.attention_split_chunk(ctx.n_single, self.kv_heads, self.head_dim, ctx.max_seq_len, keys)
