@@ -29,13 +29,15 @@ __global__ void group_rmsnorm_kernel(T* __restrict__ out, const float* __restric
     float* partial = inv + groups;
     int r = rows ? rows[blockIdx.x] : blockIdx.x;
     const float* src = x + (size_t)r * D;
-    float wi[MAX_STREAMS];
-#pragma unroll
-    for (int s = 0; s < MAX_STREAMS; ++s) wi[s] = s < n_streams ? (w_in ? w_in[s] : 1.0f) : 0.0f;
+    bool plain = n_streams == 1 && w_in == nullptr;
     for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        float u = wi[0] * src[d];
-        if (n_streams == 1 && w_in == nullptr) u = src[d];
-        for (int s = 1; s < n_streams; ++s) u = fmaf(wi[s], src[(size_t)s * stream_stride + d], u);
+        float v[MAX_STREAMS];                   // (every stream's value is asked for before the first is used)
+#pragma unroll
+        for (int s = 0; s < MAX_STREAMS; ++s) v[s] = s < n_streams ? src[(size_t)s * stream_stride + d] : 0.0f;
+        float u = plain ? v[0] : (w_in ? w_in[0] : 1.0f) * v[0];
+#pragma unroll
+        for (int s = 1; s < MAX_STREAMS; ++s)
+            if (s < n_streams) u = fmaf(w_in ? w_in[s] : 1.0f, v[s], u);
         row[d] = u;
     }
     __syncthreads();

@@ -66,6 +66,7 @@ class StepContext:
         self.block_tables: List[torch.Tensor] = []
         self.entries: List[Tuple[int, int, int]] = []   # host copy: (slot, start, count)
         self.max_seq_len = 0                            # largest start + count among the entries
+        self.longest = 0                                # the most tokens an entry brings
         self.n_single = 0                               # entries that bring one token
         self.single_lens: List[int] = []                # their lengths with that token
         self._keys_seen = {}
@@ -254,6 +255,7 @@ class StepRunner:
         c.entries = entries
         c.wants_every_row = bool(wants_all)       # the wanted rows are the step's rows, each once and in order
         c.max_seq_len = max(start + count for _, start, count in entries)
+        c.longest = max(count for _, _, count in entries)
         c.single_lens = [start + 1 for _, start, count in entries if count == 1]
         c.n_single = len(c.single_lens)
         c._keys_seen = {}

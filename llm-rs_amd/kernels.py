@@ -193,9 +193,9 @@ class HipKernels(Kernels):
             "llmrs_streams_mix": [V, V, ctypes.c_long, I, V, V, V, ctypes.c_long],
             "llmrs_streams_copy_first": [V, V, ctypes.c_long, I, ctypes.c_long],
             "llmrs_qkv_finish": [V, I, V, I, V, V, I, V, V, V, I, I, I, I, I, I, I, I, F],
-            "llmrs_mingru_scan": [V, I, V, I, V, V, V, ctypes.c_long, V, V, I, I, V, I],
+            "llmrs_mingru_scan": [V, I, V, I, V, V, V, ctypes.c_long, V, V, I, I, V, I, I, V],
             "llmrs_causal_conv_silu": [V, I, V, I, V, V, V, ctypes.c_long, V, V, V, I, I, I, I, V, I],
-            "llmrs_selective_scan": [V, I, V, I, V, I, I, I, V, I, V, V, V, V, I, V, ctypes.c_long, V, V, V, I, I, I, V, I],
+            "llmrs_selective_scan": [V, I, V, I, V, I, I, I, V, I, V, V, V, V, I, V, ctypes.c_long, V, V, V, I, I, I, I, V, I, I, V],
         }
         for name, args in sigs.items():
             fn = getattr(lib, name)
@@ -213,6 +213,13 @@ class HipKernels(Kernels):
         # steps are not recorded into graphs, so that each kernel can be seen by itself
         self.times: Optional[KernelTimes] = KernelTimes() if os.environ.get("LLM_PERF") else None
         lib.llmrs_attention_scratch_floats.restype = ctypes.c_long
+        lib.llmrs_scan_places.argtypes = [ctypes.c_long, ctypes.c_long]
+        lib.llmrs_scan_places.restype = ctypes.c_long
+        lib.llmrs_scan_chunk.argtypes = []
+        lib.llmrs_scan_chunk.restype = I
+        self.scan_chunk = lib.llmrs_scan_chunk()
+        lib.llmrs_scan_set_chunk.argtypes = [I]
+        lib.llmrs_scan_set_chunk.restype = I
         lib.llmrs_attention_scratch_floats.argtypes = [I, I, I, I, I, I]
         lib.llmrs_attention_split_chunk.restype = I
         lib.llmrs_attention_split_chunk.argtypes = [ctypes.c_long, I, I, I, ctypes.c_long]
@@ -501,17 +508,32 @@ class HipKernels(Kernels):
                   self._stream(), _code(q.dtype), _p(sums), sums.stride(0), _p(bias), _p(q), q.stride(0), _p(slot_map),
                   _p(k_cache), _p(v_cache), T, n_heads, n_kv_heads, head_dim, v_dim, page_size, num_pages, int(write_kv), float(eps))
 
-    def mingru_scan(self, sums: torch.Tensor, bias_z, bias_c, state: torch.Tensor, q_starts, slots, width: int, out: torch.Tensor) -> None:
-        """sums [T, gate | candidate | output gate] float32; state [slots, width] float32, read and left; out [T, width]."""
+    def scan_carry_floats(self, n_tokens: int, n_entries: int, longest: int, per_place: int) -> int:
+        """Room (in floats) for what the chunks of a recurrence hand on, `per_place` floats for each chunk's place;
+        0 when no entry of the step is long enough to be cut."""
+        return int(self.lib.llmrs_scan_places(n_tokens, n_entries)) * per_place if longest > self.scan_chunk else 0
+
+    def scan_set_chunk(self, tokens: int) -> None:
+        """The chunk length of the recurrences: 32 or 64 tokens, or 0 for the launcher's own choice."""
+        if self.lib.llmrs_scan_set_chunk(int(tokens)):
+            raise KernelError(self.lib.llmrs_hip_error().decode())
+
+    def mingru_scan(self, sums: torch.Tensor, bias_z, bias_c, state: torch.Tensor, q_starts, slots, width: int, out: torch.Tensor,
+                    longest: int = 0, carry: Optional[torch.Tensor] = None) -> None:
+        """sums [T, gate | candidate | output gate] float32; state [slots, width] float32, read and left; out [T, width].
+        longest: the most tokens an entry brings; with `carry` (scan_carry_floats(T, entries, longest, 2 * width)
+        floats) entries longer than a chunk run in chunks side by side."""
         assert sums.dtype == torch.float32 and sums.stride(1) == 1 and sums.shape[1] == 3 * width and out.stride(1) == 1
         assert state.dtype == torch.float32 and state.stride(-1) == 1 and state.shape[1] >= width and out.shape == (sums.shape[0], width)
         assert q_starts.dtype == slots.dtype == torch.int32 and q_starts.numel() == slots.numel() + 1
         for b in (bias_z, bias_c):
             assert b is None or (b.dtype == torch.float32 and b.numel() == width)
         T = sums.shape[0]
+        assert carry is None or (carry.dtype == torch.float32 and carry.is_contiguous()
+                                 and carry.numel() >= self.scan_carry_floats(T, slots.numel(), longest, 2 * width))
         self._run(f"mingru_scan {T}x{width}", T * width * (12 + out.element_size()), 12 * T * width, None, self.lib.llmrs_mingru_scan,
                   self._stream(), _code(out.dtype), _p(sums), sums.stride(0), _p(bias_z), _p(bias_c), _p(state), state.stride(0),
-                  _p(q_starts), _p(slots), slots.numel(), width, _p(out), out.stride(0))
+                  _p(q_starts), _p(slots), slots.numel(), width, _p(out), out.stride(0), int(longest), _p(carry))
 
     def causal_conv_silu(self, sums: torch.Tensor, taps: torch.Tensor, bias, state: torch.Tensor, q_starts, slots, token_entry,
                          channels: int, out: torch.Tensor) -> None:
@@ -528,10 +550,12 @@ class HipKernels(Kernels):
 
     def selective_scan(self, x: torch.Tensor, bc: torch.Tensor, off_b: int, off_c: int, dt: torch.Tensor, dt_bias, A: torch.Tensor,
                        D: torch.Tensor, gate: torch.Tensor, state: torch.Tensor, q_starts, slots, out: torch.Tensor,
-                       ypart: Optional[torch.Tensor] = None) -> None:
+                       ypart: Optional[torch.Tensor] = None, longest: int = 0, carry: Optional[torch.Tensor] = None) -> None:
         """S[c, n] <- exp(step_c A[c, n]) S[c, n] + step_c x_c B_n, y_c = sum_n S[c, n] C_n + D_c x_c, out = y * silu(gate),
         step = softplus(dt + dt_bias); x, bc (B at column off_b, C at off_c) and out in the activation type, dt and gate
-        float32 [T, channels], state [slots, >= channels * states] float32, read and left."""
+        float32 [T, channels], state [slots, >= channels * states] float32, read and left.  longest: the most tokens an
+        entry brings; with `carry` (scan_carry_floats(T, entries, longest, (states + 1) * channels) floats) entries
+        longer than a chunk run in chunks side by side."""
         C, N = A.shape
         T = x.shape[0]
         assert x.dtype == bc.dtype == out.dtype and x.stride(1) == bc.stride(1) == out.stride(1) == 1 and x.shape[1] == C
@@ -539,10 +563,13 @@ class HipKernels(Kernels):
         assert dt.stride(1) == gate.stride(1) == 1 and dt.shape == (T, C) and gate.shape == (T, C) and out.shape == (T, C)
         assert state.stride(-1) == 1 and state.shape[1] >= C * N and (dt_bias is None or (dt_bias.dtype == torch.float32 and dt_bias.numel() == C))
         assert ypart is None or (ypart.dtype == torch.float32 and ypart.is_contiguous() and ypart.numel() >= T * C)
+        assert bc.shape[0] == T and q_starts.dtype == slots.dtype == torch.int32 and q_starts.numel() == slots.numel() + 1
+        assert carry is None or (carry.dtype == torch.float32 and carry.is_contiguous()
+                                 and carry.numel() >= self.scan_carry_floats(T, slots.numel(), longest, (N + 1) * C))
         self._run(f"selective_scan {T}x{C}x{N}", T * (C * (8 + 2 * x.element_size()) + 2 * N * x.element_size()), 7 * T * C * N, None,
                   self.lib.llmrs_selective_scan, self._stream(), _code(x.dtype), _p(x), x.stride(0), _p(bc), bc.stride(0), int(off_b),
                   int(off_c), _p(dt), dt.stride(0), _p(dt_bias), _p(A), _p(D), _p(gate), gate.stride(0), _p(state), state.stride(0),
-                  _p(ypart), _p(q_starts), _p(slots), slots.numel(), C, N, _p(out), out.stride(0))
+                  _p(ypart), _p(q_starts), _p(slots), slots.numel(), T, C, N, _p(out), out.stride(0), int(longest), _p(carry))
 
     def argmax_rows(self, logits: torch.Tensor, out: torch.Tensor, scratch: Optional[torch.Tensor] = None) -> None:
         """`scratch`: 256 bytes per row let several blocks share a long row."""

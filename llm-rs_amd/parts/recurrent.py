@@ -62,7 +62,9 @@ class MinGRU(Mixer):
         sums = ctx.workspace("mingru.sums", (T, 3 * self.width), torch.float32)
         k.gemm(x, self.w_in, sums, EPI_STORE_F32, ctx.gemm_workspace(x, self.w_in))
         gated = ctx.workspace("mingru.gated", (T, self.width), self.dtype)
-        k.mingru_scan(sums, self.bias_z, self.bias_c, cache.state, ctx.q_starts, ctx.slots, self.width, gated)
+        need = k.scan_carry_floats(T, ctx.n_entries, ctx.longest, 2 * self.width)
+        carry = ctx.workspace("scan.carry", (need,), torch.float32) if need else None
+        k.mingru_scan(sums, self.bias_z, self.bias_c, cache.state, ctx.q_starts, ctx.slots, self.width, gated, ctx.longest, carry)
         k.gemm(gated, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(gated, self.w_o))
         ctx.note_left(h, None)
 
@@ -127,7 +129,10 @@ class Mamba1(Mixer):
         k.gemm(d, self.w_dt, dt, EPI_STORE_F32, ctx.gemm_workspace(d, self.w_dt))
         y = ctx.workspace("mamba.y", (T, C), self.dtype)
         ypart = ctx.workspace("mamba.ypart", (T, C), torch.float32) if N > 64 else None
-        k.selective_scan(xc, dbc, R, R + N, dt, self.dt_bias, self.A, self.D, sums[:, C:], scan_state, ctx.q_starts, ctx.slots, y, ypart)
+        need = k.scan_carry_floats(T, ctx.n_entries, ctx.longest, (N + 1) * C)
+        carry = ctx.workspace("scan.carry", (need,), torch.float32) if need else None
+        k.selective_scan(xc, dbc, R, R + N, dt, self.dt_bias, self.A, self.D, sums[:, C:], scan_state, ctx.q_starts, ctx.slots, y, ypart,
+                         ctx.longest, carry)
         k.gemm(y, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(y, self.w_o))
         ctx.note_left(h, None)
 

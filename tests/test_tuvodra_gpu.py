@@ -223,6 +223,37 @@ def test_the_first_token_is_still_in_the_state_after_hundreds(layer, dtype):
         check_rows(replay(eng, steps), exact, requests, allowed, name)
 
 
+@pytest.fixture
+def chunk_length(request):
+    from llm_rs_amd.kernels import kernels
+    kernels().scan_set_chunk(request.param)
+    yield request.param
+    kernels().scan_set_chunk(0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("chunk_length", [32, 64], indirect=True)
+@pytest.mark.parametrize("layer", ["mingru", "mamba1", "mamba1 many states"])
+def test_portions_longer_than_a_chunk_of_the_recurrences(layer, chunk_length, dtype):
+    """Entries of 64 tokens and more run their recurrences in chunks side by side: lengths at the chunks' edges, side
+    by side with short entries in one step, portions that start in the middle of a sequence, and a state (slow gates,
+    slow decay) in which everything before still counts."""
+    mixer = {"mingru": mingru(70), "mamba1": mamba1(72, 5, 4, 3), "mamba1 many states": mamba1(10, 70, 2, 2)}[layer]
+    cfg = one_layer(mixer, width=32, vocab=40)
+    typed, tensors = make_model(cfg, seed=8, change=long_memory)
+    lengths = {"a": 64, "b": 65, "c": 128, "d": 129, "e": 200, "f": 1, "g": 3, "h": 321}
+    requests = {r: random_tokens(40, n, 20 + i) for i, (r, n) in enumerate(lengths.items())}
+    exact = reference(cfg, tensors, requests)
+    allowed = allowed_error(dtype, cfg, tensors, requests, exact)
+    together = [{"step": 0, "entries": [{"id": r, "tokens": t, "want": list(range(len(t)))} for r, t in requests.items()], "end": list(requests)}]
+    eng = engine_for(typed, tensors, dtype, 16, sum(-(-n // 16) * 16 for n in lengths.values()), max_requests=8)
+    check_rows(replay(eng, together), exact, requests, allowed, "together")
+    for name, steps in {"whole": whole(requests), "portions": portions(requests, (3, 66, 2, 127, 64, 65)),
+                        "mixed": mixed(requests, live=3, prefill_sizes=(70, 2, 130))}.items():
+        eng = engine_for(typed, tensors, dtype, 16, live_token_need(steps, 64))
+        check_rows(replay(eng, steps), exact, requests, allowed, name)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_a_slot_used_again_starts_from_nothing(dtype):
     cfg = CONFIGS["plain"]
