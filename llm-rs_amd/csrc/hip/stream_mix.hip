@@ -18,27 +18,81 @@ struct StreamWeights {
     float w[MAX_STREAMS];
 };
 
+__device__ __forceinline__ void store4(float* p, const float (&v)[4]) { *(float4*)p = make_float4(v[0], v[1], v[2], v[3]); }
+__device__ __forceinline__ void store4(bf16* p, const float (&v)[4]) {
+    typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+    bf16x4_t t;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) t[j] = (bf16)v[j];
+    *(bf16x4_t*)p = t;
+}
+
 // One block per output row.  The combined row lives in LDS between the sums of squares and the scaling.
-template <class T>
-__global__ void group_rmsnorm_kernel(T* __restrict__ out, const float* __restrict__ x, size_t stream_stride, int n_streams,
+// MIX: what a sublayer gave (y) goes into the streams first, as streams_mix_kernel does it and with the same sums in
+// the same order; the row that is normed is combined from the new streams, which are written back on the way.
+// SMAX: a bound of n_streams that the loops over streams are unrolled to.  A thread takes four neighbouring
+// features at a time where rows are a multiple of four long (`wide`), else one.
+template <class T, bool MIX, int SMAX>
+__global__ void group_rmsnorm_kernel(T* __restrict__ out, float* __restrict__ x, size_t stream_stride, int n_streams,
                                      const float* __restrict__ w_in, const float* __restrict__ weight,
                                      const int* __restrict__ rows, int D, int groups, float eps,
-                                     float* __restrict__ zero, float* __restrict__ combined) {
-    extern __shared__ float row[];           // [D], then [groups] inverse roots, then [16] partial sums
+                                     float* zero, float* __restrict__ combined,
+                                     const float* __restrict__ mix, const float* __restrict__ w_out, const float* y, int wide) {
+    extern __shared__ float row[];           // [D], then [groups] inverse roots, then [16] partial sums, then the mix
     float* inv = row + D;
     float* partial = inv + groups;
+    float* m = partial + 16;                 // [MAX_STREAMS * MAX_STREAMS] mix, [MAX_STREAMS] w_out
     int r = rows ? rows[blockIdx.x] : blockIdx.x;
-    const float* src = x + (size_t)r * D;
+    float* src = x + (size_t)r * D;
+    if (MIX) {
+        for (int i = threadIdx.x; i < n_streams * n_streams; i += blockDim.x) m[i] = mix[i];
+        for (int i = threadIdx.x; i < n_streams; i += blockDim.x) m[MAX_STREAMS * MAX_STREAMS + i] = w_out[i];
+        __syncthreads();
+    }
     bool plain = n_streams == 1 && w_in == nullptr;
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        float v[MAX_STREAMS];                   // (every stream's value is asked for before the first is used)
+    int each = wide ? 4 : 1;
+    for (int d = threadIdx.x * each; d < D; d += blockDim.x * each) {
+        float v[SMAX][4];                       // (every stream's values are asked for before the first is used)
 #pragma unroll
-        for (int s = 0; s < MAX_STREAMS; ++s) v[s] = s < n_streams ? src[(size_t)s * stream_stride + d] : 0.0f;
-        float u = plain ? v[0] : (w_in ? w_in[0] : 1.0f) * v[0];
+        for (int s = 0; s < SMAX; ++s) {
+            v[s][0] = v[s][1] = v[s][2] = v[s][3] = 0.0f;
+            if (s < n_streams) {
+                if (wide) load4(src + (size_t)s * stream_stride + d, v[s]);
+                else v[s][0] = src[(size_t)s * stream_stride + d];
+            }
+        }
+        if (MIX) {
+            float yy[4] = {0.0f, 0.0f, 0.0f, 0.0f}, old[SMAX][4];
+            if (wide) load4(y + (size_t)r * D + d, yy);
+            else yy[0] = y[(size_t)r * D + d];
 #pragma unroll
-        for (int s = 1; s < MAX_STREAMS; ++s)
-            if (s < n_streams) u = fmaf(w_in ? w_in[s] : 1.0f, v[s], u);
-        row[d] = u;
+            for (int s = 0; s < SMAX; ++s)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) old[s][j] = v[s][j];
+#pragma unroll
+            for (int to = 0; to < SMAX; ++to) {
+                if (to < n_streams) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        float nv = m[to] * old[0][j];
+#pragma unroll
+                        for (int s = 1; s < SMAX; ++s)
+                            if (s < n_streams) nv = fmaf(m[s * n_streams + to], old[s][j], nv);
+                        v[to][j] = fmaf(m[MAX_STREAMS * MAX_STREAMS + to], yy[j], nv);
+                    }
+                    if (wide) store4(src + (size_t)to * stream_stride + d, v[to]);
+                    else src[(size_t)to * stream_stride + d] = v[to][0];
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float u = plain ? v[0][j] : (w_in ? w_in[0] : 1.0f) * v[0][j];
+#pragma unroll
+            for (int s = 1; s < SMAX; ++s)
+                if (s < n_streams) u = fmaf(w_in ? w_in[s] : 1.0f, v[s][j], u);
+            if (j < each) row[d + j] = u;
+        }
     }
     __syncthreads();
     int gs = D / groups, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
@@ -59,10 +113,23 @@ __global__ void group_rmsnorm_kernel(T* __restrict__ out, const float* __restric
         __syncthreads();
     }
     T* dst = out + (size_t)blockIdx.x * D;
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        dst[d] = from_f32<T>(row[d] * inv[d / gs] * weight[d]);
-        if (zero) zero[(size_t)blockIdx.x * D + d] = 0.0f;
-        if (combined) combined[(size_t)blockIdx.x * D + d] = row[d];
+    for (int d = threadIdx.x * each; d < D; d += blockDim.x * each) {
+        float o[4], c[4], z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int dj = j < each ? d + j : d;
+            c[j] = row[dj];
+            o[j] = c[j] * inv[dj / gs] * weight[dj];
+        }
+        if (wide) {
+            store4(dst + d, o);
+            if (zero) store4(zero + (size_t)blockIdx.x * D + d, z);
+            if (combined) store4(combined + (size_t)blockIdx.x * D + d, c);
+        } else {
+            dst[d] = from_f32<T>(o[0]);
+            if (zero) zero[(size_t)blockIdx.x * D + d] = 0.0f;
+            if (combined) combined[(size_t)blockIdx.x * D + d] = c[0];
+        }
     }
 }
 
@@ -102,24 +169,30 @@ __global__ void streams_copy_first_kernel(float* __restrict__ x, size_t stream_s
 // out[i, :] = weight * groupnorm(sum_s w_in[s] x[s][rows[i] or i, :]) in the type `dtype` says.
 // zero: if given, [n_rows, D] 32-bit that is cleared on the way (room for a sublayer to add its result into);
 // combined: if given, [n_rows, D] 32-bit that gets the combined rows before the norm.
-extern "C" int llmrs_group_rmsnorm(hipStream_t stream, int dtype, void* out, const float* x, long stream_stride, int n_streams,
+// mix, w_out, y: if given (all three; no `rows` then), x <- streams_mix(x, mix, w_out, y) first, in the same launch;
+// y may be the memory that `zero` clears.
+extern "C" int llmrs_group_rmsnorm(hipStream_t stream, int dtype, void* out, float* x, long stream_stride, int n_streams,
                                    const float* w_in, const float* weight, const int* rows, int n_rows, int D, int groups,
-                                   float eps, float* zero, float* combined) {
+                                   float eps, float* zero, float* combined, const float* mix, const float* w_out, const float* y) {
     LLMRS_REQUIRE(n_rows >= 0 && D > 0, "group_rmsnorm: bad sizes rows=%d D=%d", n_rows, D);
     LLMRS_REQUIRE(eps > 0.0f, "group_rmsnorm: eps must be positive, got %g", eps);
     LLMRS_REQUIRE(groups > 0 && groups <= MAX_NORM_GROUPS && D % groups == 0, "group_rmsnorm: %d features do not fall into %d equal groups (at most %d)", D, groups, MAX_NORM_GROUPS);
     LLMRS_REQUIRE(n_streams >= 1 && n_streams <= MAX_STREAMS, "group_rmsnorm: %d streams (at most %d)", n_streams, MAX_STREAMS);
-    LLMRS_REQUIRE(D <= 15360, "group_rmsnorm: rows of %d features do not fit the block's memory", D);
+    LLMRS_REQUIRE(D <= 15000, "group_rmsnorm: rows of %d features do not fit the block's memory", D);
+    LLMRS_REQUIRE(mix == nullptr || (w_out != nullptr && y != nullptr && rows == nullptr), "group_rmsnorm: a mix needs its weights and every row in place");
     if (n_rows == 0) return 0;
     if (dtype != LLMRS_F32 && dtype != LLMRS_BF16) return llmrs_fail("group_rmsnorm: unknown dtype %d", dtype);
-    int threads = D > 4096 ? 1024 : 256;
-    size_t lds = (size_t)(D + groups + 16) * sizeof(float);
-    if (dtype == LLMRS_F32)
-        group_rmsnorm_kernel<float><<<n_rows, threads, lds, stream>>>((float*)out, x, (size_t)stream_stride, n_streams, w_in, weight,
-                                                                      rows, D, groups, eps, zero, combined);
-    else
-        group_rmsnorm_kernel<bf16><<<n_rows, threads, lds, stream>>>((bf16*)out, x, (size_t)stream_stride, n_streams, w_in, weight,
-                                                                     rows, D, groups, eps, zero, combined);
+    int wide = D % 4 == 0 && stream_stride % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)y & 15) == 0
+               && ((uintptr_t)zero & 15) == 0 && ((uintptr_t)combined & 15) == 0;
+    int threads = D > 8192 ? 1024 : D > 2048 ? 512 : 256;
+    size_t lds = (size_t)(D + groups + 16 + MAX_STREAMS * MAX_STREAMS + MAX_STREAMS) * sizeof(float);
+#define NORM(T, MIX, SMAX) group_rmsnorm_kernel<T, MIX, SMAX><<<n_rows, threads, lds, stream>>>((T*)out, x, (size_t)stream_stride, n_streams, w_in, weight, \
+                                                                                          rows, D, groups, eps, zero, combined, mix, w_out, y, wide)
+#define BY_STREAMS(T, MIX) do { if (n_streams <= 4) NORM(T, MIX, 4); else NORM(T, MIX, MAX_STREAMS); } while (0)
+    if (dtype == LLMRS_F32) { if (mix) BY_STREAMS(float, true); else BY_STREAMS(float, false); }
+    else { if (mix) BY_STREAMS(bf16, true); else BY_STREAMS(bf16, false); }
+#undef BY_STREAMS
+#undef NORM
     LLMRS_LAUNCH_CHECK("group_rmsnorm");
     return 0;
 }

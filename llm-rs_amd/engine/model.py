@@ -113,6 +113,7 @@ class Model:
         [n_want, vocab] at the wanted rows, or None when none is wanted."""
         k = kernels()
         T = ctx.n_tokens
+        ctx.drop_streams_mix()          # (a step that ended in an error may have left one)
         if self.streamed:
             # [streams, T, hidden]: every copy starts as the embedding; blocks read and write all of them
             h = ctx.workspace("model.h", (self.streams, T, self.spec.hidden_size), torch.float32)
@@ -134,9 +135,11 @@ class Model:
             if not block.keeps_left_current:
                 ctx.note_left(h, None)
             if ctx.after_run is not None:
+                ctx.flush_streams()
                 ctx.after_run(i, h)
         ctx.norm_after_block = ctx.upcoming_norm = None
         if ctx.n_want == 0:
+            ctx.flush_streams()
             return None
         # Norm only the wanted rows, then the output matrix: the reference norms all
         # rows and gathers after (src/arch/llama.rs:135-139), which is the same numbers.

@@ -86,6 +86,33 @@ class StepContext:
         # For whoever wants to look at the stream between layers (debugging, tests): called as after_run(run, h)
         # after every run of the schedule.  None in service; a step with it set is never recorded.
         self.after_run = None
+        self._streams_mix = None        # (streams, mix, w_out, y) of a mix that is still to be done
+
+    # A block on several streams leaves its last mix to the norm that reads the streams next (one launch, one pass
+    # over the streams less).  Whoever else reads them calls flush_streams() first.
+    def defer_streams_mix(self, hs, mix, w_out, y) -> None:
+        self.flush_streams()
+        self._streams_mix = (hs, mix, w_out, y)
+
+    def take_streams_mix(self, hs):
+        """The (mix, w_out, y) still to be done on `hs`, now the caller's to do; None when there is none."""
+        pending = self._streams_mix
+        if pending is None:
+            return None
+        if pending[0].data_ptr() != hs.data_ptr() or pending[0].shape != hs.shape:
+            self.flush_streams()
+            return None
+        self._streams_mix = None
+        return pending[1:]
+
+    def drop_streams_mix(self) -> None:
+        self._streams_mix = None
+
+    def flush_streams(self) -> None:
+        pending, self._streams_mix = self._streams_mix, None
+        if pending is not None:
+            from ..kernels import kernels
+            kernels().streams_mix(*pending)
 
     def workspace(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         return self._runner.workspace(name, shape, dtype)

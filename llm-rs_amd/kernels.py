@@ -189,7 +189,7 @@ class HipKernels(Kernels):
             "llmrs_sample_rows": [V, V, I, I, I, V, V],
             "llmrs_place_ids": [V, V, I, V, V, V, I, I, I],
             "llmrs_attention_ext": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, ctypes.c_long, I, I, V, V],
-            "llmrs_group_rmsnorm": [V, I, V, V, ctypes.c_long, I, V, V, V, I, I, I, F, V, V],
+            "llmrs_group_rmsnorm": [V, I, V, V, ctypes.c_long, I, V, V, V, I, I, I, F, V, V, V, V, V],
             "llmrs_streams_mix": [V, V, ctypes.c_long, I, V, V, V, ctypes.c_long],
             "llmrs_streams_copy_first": [V, V, ctypes.c_long, I, ctypes.c_long],
             "llmrs_qkv_finish": [V, I, V, I, V, V, I, V, V, V, I, I, I, I, I, I, I, I, F],
@@ -460,10 +460,11 @@ class HipKernels(Kernels):
     # out[i, :] = weight * groupnorm(sum_s w_in[s] * x[s][rows[i] or i, :]); x: [T, D] or [S, T, D] float32
     def group_rmsnorm(self, out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, groups: int,
                       rows: Optional[torch.Tensor] = None, w_in: Optional[torch.Tensor] = None,
-                      zero: Optional[torch.Tensor] = None, combined: Optional[torch.Tensor] = None) -> None:
+                      zero: Optional[torch.Tensor] = None, combined: Optional[torch.Tensor] = None, mix=None) -> None:
         """The RMS norm in `groups` equal consecutive parts of the row.  `x` with three dimensions is several streams,
         combined with the weights `w_in` (None: summed) before the norm.  `zero` [n, D] float32 is cleared on the way,
-        `combined` [n, D] float32 gets the combined rows."""
+        `combined` [n, D] float32 gets the combined rows.  `mix` = (mix [S, S], w_out [S], y [n, D]): `streams_mix`
+        of these runs on x first, in the same launch (every row, no `rows`); y may be `zero`."""
         assert x.dtype == torch.float32 and weight.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous()
         S = x.shape[0] if x.dim() == 3 else 1
         D, n = x.shape[-1], out.shape[0]
@@ -472,10 +473,17 @@ class HipKernels(Kernels):
         assert w_in is None or (w_in.dtype == torch.float32 and w_in.numel() == S)
         for extra in (zero, combined):
             assert extra is None or (extra.dtype == torch.float32 and extra.is_contiguous() and tuple(extra.shape) == (n, D))
-        self._run(f"group_rmsnorm {n}x{D}" + (f" of {S} streams" if S > 1 else ""), n * D * (4 * S + out.element_size()) + D * 4,
-                  (2 * S + 5) * n * D, None, self.lib.llmrs_group_rmsnorm, self._stream(), _code(out.dtype), _p(out), _p(x),
+        m = w_out = y = None
+        if mix is not None:
+            m, w_out, y = mix
+            assert rows is None and x.dim() == 3 and m.dtype == w_out.dtype == y.dtype == torch.float32
+            assert tuple(m.shape) == (S, S) and m.is_contiguous() and w_out.numel() == S and y.is_contiguous() and tuple(y.shape) == (n, D)
+        traffic = n * D * (4 * S + out.element_size()) + D * 4 + (n * D * 4 * (S + 1) if mix is not None else 0)
+        self._run(f"group_rmsnorm {n}x{D}" + (f" of {S} streams" if S > 1 else "") + (" after their mix" if mix is not None else ""),
+                  traffic, (2 * S + 5 + (2 * S * S if mix is not None else 0)) * n * D, None, self.lib.llmrs_group_rmsnorm,
+                  self._stream(), _code(out.dtype), _p(out), _p(x),
                   x.stride(0) if x.dim() == 3 else 0, S, _p(w_in), _p(weight), _p(rows), n, D, int(groups), float(eps),
-                  _p(zero), _p(combined))
+                  _p(zero), _p(combined), _p(m), _p(w_out), _p(y))
 
     # x[r] = sum_s mix[s, r] * x[s] + w_out[r] * y, all streams at once from the old ones; x: [S, T, D] float32
     def streams_mix(self, x: torch.Tensor, mix: torch.Tensor, w_out: torch.Tensor, y: torch.Tensor) -> None:

@@ -38,7 +38,9 @@ class HyperConnection(Part):
         return {self.name("in"): self.w_in.cpu(), self.name("out"): self.w_out.cpu(), self.name("mix"): self.mix.cpu()}
 
     def write(self, ctx, hs: torch.Tensor, y: torch.Tensor) -> None:
-        kernels().streams_mix(hs, self.mix, self.w_out, y)
+        """The mix is left to whoever reads the streams next: a norm that reads every row does it in its own
+        launch; anyone else asks the context to do it first (`flush_streams`)."""
+        ctx.defer_streams_mix(hs, self.mix, self.w_out, y)
 
 
 register_connection = register_part_family("connection")

@@ -56,6 +56,7 @@ class GroupRMSNorm(Norm):
     It also reads a stream kept in several copies, combined with given weights on the way (`forward_streams`).
     `tensor`: the leaf of the weight's name ("weight"); "" when the prefix itself is the name."""
     graph_safe = True
+    FUSE_MIX_FROM_ROWS = 128
 
     def __init__(self, spec, dtype):
         super().__init__(spec, dtype)
@@ -81,7 +82,12 @@ class GroupRMSNorm(Norm):
         kernels().group_rmsnorm(out, h, self.weight, self.eps, self.groups, rows)
 
     def forward_streams(self, ctx, hs, w_in, out, rows=None, zero=None):
-        kernels().group_rmsnorm(out, hs, self.weight, self.eps, self.groups, rows, w_in=w_in, zero=zero)
+        # A mix of these streams that is still to be done runs in the norm's launch, when the norm reads every row
+        # and there are rows enough to fill the device with one block a row (the mix alone spreads a row over blocks).
+        mix = ctx.take_streams_mix(hs) if rows is None and hs.shape[1] >= self.FUSE_MIX_FROM_ROWS else None
+        if mix is None:
+            ctx.flush_streams()
+        kernels().group_rmsnorm(out, hs, self.weight, self.eps, self.groups, rows, w_in=w_in, zero=zero, mix=mix)
         return True
 
 

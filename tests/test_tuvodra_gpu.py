@@ -290,6 +290,18 @@ def test_long_decoding_with_recorded_steps(dtype):
     assert eng.runner.graph_replays > 100           # the single-token steps were recorded and replayed
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("streams,width,groups", [(5, 42, 3), (2, 40, 2), (4, 36, 1), (1, 44, 2)])
+def test_steps_of_many_rows_mix_the_streams_inside_the_next_norm(streams, width, groups, dtype):
+    """From 128 rows on, a sublayer's mix of the streams runs in the launch of the norm that reads them next: rows of
+    a length that is and is not a multiple of four, few and many streams, steps just below and above that bound."""
+    cfg = config(width, 53, streams, groups, 1.5, [mingru(24, ff=32), attention(2, 1, 8, 8, 0.5, 11), mamba1(16, 3, 2, 2, ff=20)])
+    typed, tensors = make_model(cfg, seed=streams)
+    requests = {"a": random_tokens(53, 127, 1), "b": random_tokens(53, 128, 2), "c": random_tokens(53, 300, 3)}
+    run_regimes(cfg, typed, tensors, dtype, 16, requests,
+                {"whole": whole(requests), "portions": portions(requests, (128, 2, 129, 41))})
+
+
 # ---- generation through the scheduler --------------------------------------------------------------------------------
 
 def plain_greedy(cfg, tensors, prompt, n):
