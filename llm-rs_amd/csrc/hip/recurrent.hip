@@ -93,7 +93,21 @@ __global__ void mingru_carry_kernel(const float* __restrict__ state, long state_
     if (chunks <= 0) return;
     size_t place = (size_t)(q0 / chunk + e);
     float s = state[(size_t)slots[e] * state_stride + c];
-    for (int k = 0; k + 1 < chunks; ++k, ++place) {
+    int k = 0;
+    for (; k + SCAN_LOADS < chunks; k += SCAN_LOADS, place += SCAN_LOADS) {     // (what SCAN_LOADS chunks left, fetched together)
+        float end[SCAN_LOADS], keep[SCAN_LOADS];
+#pragma unroll
+        for (int i = 0; i < SCAN_LOADS; ++i) {
+            end[i] = carry[(place + i) * 2 * W + c];
+            keep[i] = carry[((place + i) * 2 + 1) * W + c];
+        }
+#pragma unroll
+        for (int i = 0; i < SCAN_LOADS; ++i) {
+            carry[(place + i) * 2 * W + c] = s;
+            s = fmaf(keep[i], s, end[i]);
+        }
+    }
+    for (; k + 1 < chunks; ++k, ++place) {
         float* p = carry + place * 2 * W + c;
         float end = p[0], keep = p[W];
         p[0] = s;

@@ -328,3 +328,47 @@ def test_greedy_generation_through_the_scheduler(which):
             if a != b:
                 assert margins[i] < 1e-4, (prompt, i, out, want)       # a tie within rounding may fall either way
                 break
+
+
+# ---- the programs, on a model folder ----------------------------------------------------------------------------------
+
+def test_the_programs_on_a_model_folder(tmp_path):
+    """A folder with config.json and model.safetensors through `bin/trace_run` (a mixed trace under a small pool, both
+    dtypes) and through `bin/llm-rs complete` (greedy): the architecture is chosen by the file."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+    from tuvodra_cases import make_folder
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = CONFIGS["plain"]
+    folder = make_folder(tmp_path, cfg, seed=11)
+    typed, tensors = make_model(cfg, seed=11)
+    requests = {f"r{i}": random_tokens(cfg["vocab"], n, 50 + i) for i, n in enumerate([33, 2, 90, 47, 18])}
+    exact = reference(cfg, tensors, requests)
+    steps = mixed(requests, live=3)
+    text = "".join(json.dumps(s) + "\n" for s in steps)
+    for dtype in DTYPES:
+        out = tmp_path / f"out_{dtype}"
+        p = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", str(out),
+                            "--max-tokens", str(live_token_need(steps, 64))], input=text, capture_output=True, text=True, timeout=600)
+        assert p.returncode == 0, p.stderr[-2000:]
+        assert [l for l in p.stdout.split("\n") if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+        outputs = []
+        for s in steps:
+            n = sum(len(e["want"]) for e in s["entries"])
+            outputs.append(torch.from_numpy(np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(n, cfg["vocab"]).copy()) if n else None)
+        check_rows(collect(steps, outputs), exact, requests, allowed_error(dtype, cfg, tensors, requests, exact), f"trace_run {dtype}")
+    prompt = requests["r3"]
+    p = subprocess.run([sys.executable, os.path.join(root, "bin", "llm-rs"), "-m", folder, "--dtype", "float32", "--num-pages", "64", "complete",
+                        "--prompt-ids", " ".join(map(str, prompt)), "-n", "10", "--temperature", "0"], capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    got = [int(t) for t in p.stdout.split()]
+    want, margins = plain_greedy(cfg, tensors, prompt, 10)
+    for i, (a, b) in enumerate(zip(got, want)):
+        if a != b:
+            assert margins[i] < 1e-4, (i, got, want)
+            break
+    assert len(got) == 10
