@@ -547,7 +547,7 @@ def tuvodra_shape(width, heads, kv_heads, dim, ff, window, repeats, vocab=128256
              {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
                                              "mask": {"size": window}}, "mlp": {"kind": "dense", "ff": ff}}]
     return {"architecture": "Tuvodra", "vocab": vocab, "width": width, "streams": 4, "embedding": {"scale": 1.0},
-            "norm": {"eps": 1e-5, "groups": 2}, "layers": [dict(l) for _ in range(repeats) for l in three]}
+            "norm": {"eps": 1e-6, "groups": 4}, "layers": [dict(l) for _ in range(repeats) for l in three]}
 
 
 def run_tuvodra(args) -> dict:
@@ -599,7 +599,7 @@ def run_tuvodra(args) -> dict:
     line = base_line("decode_tokens_per_s", first["decode_tokens_per_s"], args.steps, args.warmup, first["decode_ms_per_step"] * 1e-3, args.dtype,
                      {"model": "Tuvodra (minGRU, selective scan, windowed attention + feed-forward, in threes) beside Llama of equal widths",
                       "global_batch": batch, "seq_len": context, "parallelism": "single GPU", "layers_run": 3 * repeats,
-                      "prefill_tokens": T, "window": args.window, "streams": 4, "page_size": 16})
+                      "prefill_tokens": T, "window": args.window, "streams": 4, "norm_groups": 4, "page_size": 16})
     line["points"] = points
     return line
 

@@ -51,6 +51,9 @@ ALONE = {
     "attention wide values": attention(3, 3, 8, 24, 1.3, 50, ff=32),
     "attention narrow values, one kv head": attention(5, 1, 20, 4, 0.05, 3),
     "attention window of one": attention(2, 2, 16, 16, 0.25, 1),
+    "attention, heads of 32 in fours": attention(4, 1, 32, 32, 0.2, 21),
+    "attention, heads of 128": attention(6, 2, 128, 128, 0.09, 70, ff=48),
+    "attention, heads of 64, window of a page": attention(8, 4, 64, 64, 0.11, 16),
 }
 
 
@@ -125,10 +128,15 @@ def sequence_with_mark(vocab, n, at, mark, seed):
     return toks
 
 
+# head shapes: values narrower than keys (the kernel for any sizes) and heads the matrix-core kernels take
+HEAD_SHAPES = {"any sizes": dict(dim=16, vdim=12, heads=2, kv_heads=1, width=32), "matrix cores": dict(dim=64, vdim=64, heads=4, kv_heads=2, width=64)}
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("window,at", [(9, 3), (16, 0), (17, 15), (33, 16), (40, 31)])
-def test_a_key_just_inside_and_just_outside_the_window(window, at, dtype):
-    cfg, typed, tensors = marked_attention_model(window)
+@pytest.mark.parametrize("shape", list(HEAD_SHAPES))
+@pytest.mark.parametrize("window,at", [(9, 3), (16, 0), (17, 15), (33, 16), (40, 31), (64, 1), (65, 30)])
+def test_a_key_just_inside_and_just_outside_the_window(window, at, shape, dtype):
+    cfg, typed, tensors = marked_attention_model(window, **HEAD_SHAPES[shape])
     toks = sequence_with_mark(cfg["vocab"], at + window + 6, at, 7, seed=window)
     requests = {"m": toks}
     exact = reference(cfg, tensors, requests)
@@ -149,8 +157,9 @@ def test_a_key_just_inside_and_just_outside_the_window(window, at, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_a_far_key_among_hundreds_across_pages(dtype):
-    cfg, typed, tensors = marked_attention_model(window=1000)
+@pytest.mark.parametrize("shape", list(HEAD_SHAPES))
+def test_a_far_key_among_hundreds_across_pages(shape, dtype):
+    cfg, typed, tensors = marked_attention_model(window=1000, **HEAD_SHAPES[shape])
     for at in (0, 15, 16, 250):
         toks = sequence_with_mark(cfg["vocab"], 600, at, 7, seed=at)
         requests = {"m": toks}
@@ -300,6 +309,40 @@ def test_steps_of_many_rows_mix_the_streams_inside_the_next_norm(streams, width,
     requests = {"a": random_tokens(53, 127, 1), "b": random_tokens(53, 128, 2), "c": random_tokens(53, 300, 3)}
     run_regimes(cfg, typed, tensors, dtype, 16, requests,
                 {"whole": whole(requests), "portions": portions(requests, (128, 2, 129, 41))})
+
+
+# ---- configurations drawn at random -----------------------------------------------------------------------------------
+
+def random_configuration(seed):
+    import random
+    r = random.Random(seed)
+    width = r.choice([24, 40, 64, 96, 136])
+    groups = r.choice([g for g in (1, 2, 3, 4, 8) if width % g == 0])
+    layers = []
+    for _ in range(r.randint(2, 5)):
+        ff = r.choice([None, None, 8 * r.randint(2, 12)])
+        kind = r.choice(["mingru", "mamba1", "attention"])
+        if kind == "mingru":
+            layers.append(mingru(4 * r.randint(3, 30), ff=ff))
+        elif kind == "mamba1":
+            layers.append(mamba1(4 * r.randint(3, 30), r.choice([1, 4, 16, 24, 33, 70]), r.randint(1, 5), r.randint(1, 9), ff=ff))
+        else:
+            kv = r.choice([1, 2, 3])
+            dim = r.choice([8, 20, 32, 64, 128])
+            vdim = r.choice([dim, dim, 4 * r.randint(1, 10)])
+            layers.append(attention(kv * r.choice([1, 2, 4]), kv, dim, vdim, r.uniform(0.05, 0.5), r.choice([1, 5, 16, 17, 31, 32, 48, 100, 500]), ff=ff))
+    return config(width, r.randint(30, 200), r.randint(1, 6), groups, r.uniform(0.5, 10.0), layers, eps=r.choice([1e-5, 1e-6, 1e-3]))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(seed, dtype):
+    cfg = random_configuration(seed)
+    typed, tensors = make_model(cfg, seed=seed)
+    requests = {f"r{i}": random_tokens(cfg["vocab"], n, 70 + i) for i, n in enumerate([150, 3, 66, 1, 35])}
+    run_regimes(cfg, typed, tensors, dtype, 16, requests,
+                {"whole": whole(requests), "decoded": tail_decoded(requests, tail=36), "portions": portions(requests, (2, 70, 3, 33)),
+                 "mixed": mixed(requests, live=3)})
 
 
 # ---- generation through the scheduler --------------------------------------------------------------------------------
