@@ -153,7 +153,7 @@ __global__ void causal_conv_state_kernel(const float* __restrict__ sums, int ld,
 }
 
 // ---- selective scan -----------------------------------------------------------------------------------------------
-// Per channel c and state n, with step = softplus(dt[t, c] + dt_bias[c]) and A[c, n] < 0:
+// Per channel c and state n, with step = softplus(dt[t, c] + dt_bias[c]) and A[c, n] < 0 (given state by channel):
 //   S[c, n] <- exp(step A[c, n]) S[c, n] + step x[t, c] B[t, n];   y = sum_n S[c, n] C[t, n] + D[c] x[t, c]
 //   out[t, c] = y * silu(gate[t, c])
 // One thread for each (entry, chunk, channel) holds NS states in registers; a channel with more states is walked in
@@ -163,10 +163,10 @@ __global__ void causal_conv_state_kernel(const float* __restrict__ sums, int ld,
 struct ScanArgs {
     const float* dt; int ld_dt;          // [T, C] sums of the step projection, 32-bit
     const float* dt_bias;                // [C]
-    const float* A;                      // [C, N], negative
+    const float* A;                      // [N, C] (state by channel), negative
     const float* D;                      // [C]
     const float* gate; int ld_gate;      // [T, C] 32-bit (the projection's second half)
-    float* state; long state_stride;     // [slots][C][N]
+    float* state; long state_stride;     // [slots][N][C]: a wave's 64 channels read a state's values side by side
     float* ypart;                        // [T, C], needed when N > NS
     float* carry;                        // [places][N][C]: the state a chunk starts from (local launch: ends with, from zero)
     float* steps;                        // [places][C]: the sum of a chunk's step sizes
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(const T* __restrict_
     }
     bool last_chunk = t1 == q1;
     if (LOCAL && last_chunk) return;
-    float* sp = a.state + (size_t)slots[e] * a.state_stride + (size_t)cc * a.N;
+    float* sp = a.state + (size_t)slots[e] * a.state_stride + cc;          // state n of this channel: sp[n * C]
     float bias = a.dt_bias ? a.dt_bias[cc] : 0.0f, Dc = a.D[cc];
     for (int n0 = 0; n0 < a.N; n0 += NS) {
         bool first = n0 == 0, last = n0 + NS >= a.N;
@@ -201,8 +201,8 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(const T* __restrict_
 #pragma unroll
         for (int n = 0; n < NS; ++n) {             // (states past the last stay zero: their B is zero)
             bool in = n0 + n < a.N;
-            S[n] = LOCAL || !in ? 0.0f : (a.chunk > 0 ? a.carry[(place * a.N + n0 + n) * a.C + cc] : sp[n0 + n]);
-            Ac[n] = in ? a.A[(size_t)cc * a.N + n0 + n] * LOG2_E : 0.0f;     // exp(step A) as 2^(step A log2 e)
+            S[n] = LOCAL || !in ? 0.0f : (a.chunk > 0 ? a.carry[(place * a.N + n0 + n) * a.C + cc] : sp[(size_t)(n0 + n) * a.C]);
+            Ac[n] = in ? a.A[(size_t)(n0 + n) * a.C + cc] * LOG2_E : 0.0f;     // exp(step A) as 2^(step A log2 e)
         }
         float step_sum = 0.0f;
         auto one = [&](int t, int r, float vdt, float xv, float vg) {
@@ -257,7 +257,7 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(const T* __restrict_
         } else if (last_chunk && live) {
 #pragma unroll
             for (int n = 0; n < NS; ++n)
-                if (n0 + n < a.N) sp[n0 + n] = S[n];
+                if (n0 + n < a.N) sp[(size_t)(n0 + n) * a.C] = S[n];
         }
     }
 }
@@ -271,7 +271,7 @@ __global__ void selective_scan_carry_kernel(const int* __restrict__ q_starts, co
     int chunks = (count + a.chunk - 1) / a.chunk;
     if (chunks <= 0) return;
     size_t place = (size_t)(q0 / a.chunk + e);
-    float s = a.state[(size_t)slots[e] * a.state_stride + (size_t)c * a.N + n], An = a.A[(size_t)c * a.N + n];
+    float s = a.state[(size_t)slots[e] * a.state_stride + (size_t)n * a.C + c], An = a.A[(size_t)n * a.C + c];
     int k = 0;
     for (; k + SCAN_LOADS < chunks; k += SCAN_LOADS, place += SCAN_LOADS) {
         float end[SCAN_LOADS], sum[SCAN_LOADS];

@@ -561,10 +561,11 @@ class HipKernels(Kernels):
                        ypart: Optional[torch.Tensor] = None, longest: int = 0, carry: Optional[torch.Tensor] = None) -> None:
         """S[c, n] <- exp(step_c A[c, n]) S[c, n] + step_c x_c B_n, y_c = sum_n S[c, n] C_n + D_c x_c, out = y * silu(gate),
         step = softplus(dt + dt_bias); x, bc (B at column off_b, C at off_c) and out in the activation type, dt and gate
-        float32 [T, channels], state [slots, >= channels * states] float32, read and left.  longest: the most tokens an
+        float32 [T, channels], A [states, channels] (transposed), state [slots, >= states * channels] float32 (state by
+        channel), read and left.  longest: the most tokens an
         entry brings; with `carry` (scan_carry_floats(T, entries, longest, (states + 1) * channels) floats) entries
         longer than a chunk run in chunks side by side."""
-        C, N = A.shape
+        N, C = A.shape
         T = x.shape[0]
         assert x.dtype == bc.dtype == out.dtype and x.stride(1) == bc.stride(1) == out.stride(1) == 1 and x.shape[1] == C
         assert dt.dtype == gate.dtype == A.dtype == D.dtype == state.dtype == torch.float32 and A.is_contiguous() and D.numel() == C
@@ -574,7 +575,8 @@ class HipKernels(Kernels):
         assert bc.shape[0] == T and q_starts.dtype == slots.dtype == torch.int32 and q_starts.numel() == slots.numel() + 1
         assert carry is None or (carry.dtype == torch.float32 and carry.is_contiguous()
                                  and carry.numel() >= self.scan_carry_floats(T, slots.numel(), longest, (N + 1) * C))
-        self._run(f"selective_scan {T}x{C}x{N}", T * (C * (8 + 2 * x.element_size()) + 2 * N * x.element_size()), 7 * T * C * N, None,
+        self._run(f"selective_scan {T}x{C}x{N}", T * (C * (8 + 2 * x.element_size()) + 2 * N * x.element_size()) + slots.numel() * C * N * 8,
+                  7 * T * C * N, None,
                   self.lib.llmrs_selective_scan, self._stream(), _code(x.dtype), _p(x), x.stride(0), _p(bc), bc.stride(0), int(off_b),
                   int(off_c), _p(dt), dt.stride(0), _p(dt_bias), _p(A), _p(D), _p(gate), gate.stride(0), _p(state), state.stride(0),
                   _p(ypart), _p(q_starts), _p(slots), slots.numel(), T, C, N, _p(out), out.stride(0), int(longest), _p(carry))

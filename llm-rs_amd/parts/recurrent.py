@@ -98,7 +98,7 @@ class Mamba1(Mixer):
         self.w_in, self.w_x, self.w_dt, self.w_o = get("in"), get("x"), get("dt"), get("out")
         self.conv, self.conv_bias, self.dt_bias, self.D = get32("conv"), get32("conv_bias"), get32("dt_bias"), get32("D")
         self.A_log = get32("A_log")
-        self.A = (-torch.exp(self.A_log)).contiguous()          # 32-bit, once
+        self.A = (-torch.exp(self.A_log)).t().contiguous()      # 32-bit, once; [state, inner] as the scan reads it
 
     def export(self):
         n = self.names
@@ -111,7 +111,7 @@ class Mamba1(Mixer):
         return super().step_weight_bytes(seen)
 
     def cache_need(self):
-        # one row per request: the scan's state [inner, state], then the convolution's last inputs [conv - 1, inner]
+        # one row per request: the scan's state [state, inner], then the convolution's last inputs [conv - 1, inner]
         return FixedState((self.inner * self.n_state + (self.taps - 1) * self.inner,), torch.float32)
 
     def forward(self, ctx, x, h, cache):
