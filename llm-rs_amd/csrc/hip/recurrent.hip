@@ -120,23 +120,45 @@ __global__ void mingru_carry_kernel(const float* __restrict__ state, long state_
 // y[t, c] = silu(bias[c] + sum_j taps[c, j] * x[t - (K - 1 - j), c]): the last tap weighs the current token.  Inputs
 // from before the step's first token come from the request's state (its last K - 1 inputs, oldest first), which is
 // zero at the start of a sequence.  x: the first C columns of `sums` [T, ld], 32-bit.
-template <class T>
+// A block takes `per_block` neighbouring tokens, one after the other (their inputs overlap).  KMAX: a bound of K
+// that the loops over taps are unrolled to, so that a token's inputs are fetched together (0: any K, one by one).
+template <class T, int KMAX>
 __global__ void causal_conv_silu_kernel(const float* __restrict__ sums, int ld, const float* __restrict__ taps,
                                         const float* __restrict__ bias, const float* __restrict__ state, long state_stride,
                                         const int* __restrict__ q_starts, const int* __restrict__ slots,
-                                        const int* __restrict__ token_entry, int C, int K, T* __restrict__ out, int ldo) {
-    int c = blockIdx.x * blockDim.x + threadIdx.x, t = blockIdx.y;
+                                        const int* __restrict__ token_entry, int n_tokens, int per_block, int C, int K,
+                                        T* __restrict__ out, int ldo) {
+    int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= C) return;
-    int e = token_entry[t];
-    int i = t - q_starts[e];                    // the token's place in its entry
-    const float* sp = state + (size_t)slots[e] * state_stride;
-    float acc = bias ? bias[c] : 0.0f;
-    for (int j = 0; j < K; ++j) {
-        int back = K - 1 - j;                   // how many tokens before this one
-        float x = i - back >= 0 ? sums[(size_t)(t - back) * ld + c] : sp[(size_t)(K - 1 + i - back) * C + c];
-        acc = fmaf(taps[(size_t)c * K + j], x, acc);
+    float b = bias ? bias[c] : 0.0f;
+    float w[KMAX > 0 ? KMAX : 1];
+#pragma unroll
+    for (int j = 0; j < KMAX; ++j) w[j] = j < K ? taps[(size_t)c * K + j] : 0.0f;
+    int t_end = min(((int)blockIdx.y + 1) * per_block, n_tokens);
+    for (int t = blockIdx.y * per_block; t < t_end; ++t) {
+        int e = token_entry[t];
+        int i = t - q_starts[e];                    // the token's place in its entry
+        const float* sp = state + (size_t)slots[e] * state_stride;
+        float acc = b;
+        if (KMAX > 0) {
+            float x[KMAX > 0 ? KMAX : 1];
+#pragma unroll
+            for (int j = 0; j < KMAX; ++j) {
+                int back = K - 1 - j;               // how many tokens before this one
+                x[j] = j >= K ? 0.0f : i - back >= 0 ? sums[(size_t)(t - back) * ld + c] : sp[(size_t)(K - 1 + i - back) * C + c];
+            }
+#pragma unroll
+            for (int j = 0; j < KMAX; ++j)
+                if (j < K) acc = fmaf(w[j], x[j], acc);
+        } else {
+            for (int j = 0; j < K; ++j) {
+                int back = K - 1 - j;
+                float x = i - back >= 0 ? sums[(size_t)(t - back) * ld + c] : sp[(size_t)(K - 1 + i - back) * C + c];
+                acc = fmaf(taps[(size_t)c * K + j], x, acc);
+            }
+        }
+        out[(size_t)t * ldo + c] = from_f32<T>(silu_f32(acc));
     }
-    out[(size_t)t * ldo + c] = from_f32<T>(silu_f32(acc));
 }
 
 // After the convolution: the state becomes the last K - 1 inputs of (old state, this step's inputs).
@@ -347,14 +369,15 @@ extern "C" int llmrs_causal_conv_silu(hipStream_t stream, int dtype, const float
     LLMRS_REQUIRE(C > 0 && K >= 1 && ld >= C && ldo >= C && state_stride >= (long)(K - 1) * C, "causal_conv: bad sizes");
     LLMRS_REQUIRE(entries_ok(q_starts, slots, n_entries) && token_entry && n_tokens >= 0 && n_tokens <= 65535 * 32, "causal_conv: bad entries");
     if (n_tokens == 0) return 0;
-    LLMRS_REQUIRE(n_tokens <= 65535, "causal_conv: %d tokens are too many for one launch", n_tokens);
-    dim3 grid(ceil_div(C, 64), n_tokens);
-    if (dtype == LLMRS_F32)
-        causal_conv_silu_kernel<float><<<grid, 64, 0, stream>>>(sums, ld, taps, bias, state, state_stride, q_starts, slots, token_entry, C, K, (float*)out, ldo);
-    else if (dtype == LLMRS_BF16)
-        causal_conv_silu_kernel<bf16><<<grid, 64, 0, stream>>>(sums, ld, taps, bias, state, state_stride, q_starts, slots, token_entry, C, K, (bf16*)out, ldo);
-    else
-        return llmrs_fail("causal_conv: unknown dtype %d", dtype);
+    int per_block = n_tokens >= 1024 ? 8 : 1, threads = n_tokens >= 1024 && C >= 256 ? 256 : 64;
+    LLMRS_REQUIRE(ceil_div(n_tokens, per_block) <= 65535, "causal_conv: %d tokens are too many for one launch", n_tokens);
+    dim3 grid(ceil_div(C, threads), ceil_div(n_tokens, per_block));
+    LLMRS_REQUIRE(dtype == LLMRS_F32 || dtype == LLMRS_BF16, "causal_conv: unknown dtype %d", dtype);
+#define CONV(T, KMAX) causal_conv_silu_kernel<T, KMAX><<<grid, threads, 0, stream>>>(sums, ld, taps, bias, state, state_stride, q_starts, slots, token_entry, n_tokens, per_block, C, K, (T*)out, ldo)
+#define BY_TAPS(T) do { if (K <= 4) CONV(T, 4); else if (K <= 8) CONV(T, 8); else CONV(T, 0); } while (0)
+    if (dtype == LLMRS_F32) BY_TAPS(float); else BY_TAPS(bf16);
+#undef BY_TAPS
+#undef CONV
     if (K > 1)
         causal_conv_state_kernel<<<dim3(ceil_div(C, 64), n_entries), 64, 0, stream>>>(sums, ld, state, state_stride, q_starts, slots, C, K);
     LLMRS_LAUNCH_CHECK("causal_conv");

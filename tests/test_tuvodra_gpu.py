@@ -47,6 +47,8 @@ ALONE = {
     "mamba1": mamba1(36, 6, 3, 4),
     "mamba1 one tap": mamba1(20, 9, 1, 2, ff=24),
     "mamba1 many states": mamba1(12, 130, 2, 5),
+    "mamba1 many taps": mamba1(20, 3, 9, 2),
+    "mamba1 six taps": mamba1(28, 2, 6, 1, ff=16),
     "attention": attention(4, 2, 12, 12, 0.4, 7),
     "attention wide values": attention(3, 3, 8, 24, 1.3, 50, ff=32),
     "attention narrow values, one kv head": attention(5, 1, 20, 4, 0.05, 3),
@@ -309,6 +311,22 @@ def test_steps_of_many_rows_mix_the_streams_inside_the_next_norm(streams, width,
     requests = {"a": random_tokens(53, 127, 1), "b": random_tokens(53, 128, 2), "c": random_tokens(53, 300, 3)}
     run_regimes(cfg, typed, tensors, dtype, 16, requests,
                 {"whole": whole(requests), "portions": portions(requests, (128, 2, 129, 41))})
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_step_of_more_than_a_thousand_tokens(dtype):
+    """Steps this long take the convolution several tokens a block: a long portion beside a short one, both continued
+    in the next step, over narrow and wide channels and several tap counts."""
+    cfg = config(32, 40, 2, 2, 2.0, [mamba1(72, 5, 4, 3), mamba1(320, 4, 3, 2), mingru(40), mamba1(24, 20, 2, 2, ff=48)])
+    typed, tensors = make_model(cfg, seed=12)
+    requests = {"a": random_tokens(40, 1100, 1), "b": random_tokens(40, 40, 2)}
+    exact = reference(cfg, tensors, requests)
+    allowed = allowed_error(dtype, cfg, tensors, requests, exact)
+    cuts = {"a": 1031, "b": 5}
+    steps = [{"step": 0, "entries": [{"id": r, "tokens": t[:cuts[r]], "want": list(range(cuts[r]))} for r, t in requests.items()], "end": []},
+             {"step": 1, "entries": [{"id": r, "tokens": t[cuts[r]:], "want": list(range(len(t) - cuts[r]))} for r, t in requests.items()], "end": list(requests)}]
+    eng = engine_for(typed, tensors, dtype, 16, 1280)
+    check_rows(replay(eng, steps), exact, requests, allowed, "two steps")
 
 
 # ---- configurations drawn at random -----------------------------------------------------------------------------------
