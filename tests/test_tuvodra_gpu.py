@@ -56,6 +56,9 @@ ALONE = {
     "attention, heads of 32 in fours": attention(4, 1, 32, 32, 0.2, 21),
     "attention, heads of 128": attention(6, 2, 128, 128, 0.09, 70, ff=48),
     "attention, heads of 64, window of a page": attention(8, 4, 64, 64, 0.11, 16),
+    "attention, heads of 64 in threes": attention(6, 2, 64, 64, 0.13, 29),
+    "attention, heads of 32, fourteen to a key head": attention(14, 1, 32, 32, 0.3, 40),
+    "attention, heads of 96": attention(4, 2, 96, 96, 0.1, 23),
 }
 
 
@@ -327,6 +330,19 @@ def test_a_step_of_more_than_a_thousand_tokens(dtype):
              {"step": 1, "entries": [{"id": r, "tokens": t[cuts[r]:], "want": list(range(len(t) - cuts[r]))} for r, t in requests.items()], "end": list(requests)}]
     eng = engine_for(typed, tensors, dtype, 16, 1280)
     check_rows(replay(eng, steps), exact, requests, allowed, "two steps")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which", ["even", "odd"])
+def test_sizes_that_are_no_multiples_of_four(which, dtype):
+    """No vector load fits these rows: every kernel's narrow path, also in steps long enough for chunks and fused norms."""
+    cfg = {"even": config(46, 51, 3, 2, 1.0, [mingru(30), mamba1(26, 3, 3, 3, ff=22), attention(3, 1, 10, 6, 0.3, 9, ff=14)]),
+           "odd": config(45, 37, 2, 3, 2.5, [attention(2, 2, 7, 5, 0.4, 6), mingru(17, ff=9), mamba1(15, 5, 2, 1)])}[which]
+    typed, tensors = make_model(cfg, seed=13)
+    requests = {"a": random_tokens(cfg["vocab"], 140, 1), "b": random_tokens(cfg["vocab"], 21, 2), "c": random_tokens(cfg["vocab"], 2, 3)}
+    run_regimes(cfg, typed, tensors, dtype, 16, requests,
+                {"whole": whole(requests), "decoded": tail_decoded(requests, tail=20), "portions": portions(requests, (3, 131, 2)),
+                 "mixed": mixed(requests, live=3)})
 
 
 # ---- configurations drawn at random -----------------------------------------------------------------------------------
