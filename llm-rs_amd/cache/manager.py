@@ -34,33 +34,46 @@ class PagedGroup:
         return self.n_layers * self.kind.bytes_per_token(self.need, self.dtype)
 
 
+def _flat(need) -> Tuple[Any, ...]:
+    """A run's needs one by one: a mixer made of several asks with a tuple."""
+    if need is None:
+        return ()
+    return tuple(n for n in need if n is not None) if isinstance(need, tuple) else (need,)
+
+
 def _group_runs(needs: Sequence[Tuple[object, Optional[int]]]):
-    """(the distinct paged needs, layers in each, (group, layer) of every run or None, the runs with per-request needs)."""
+    """(the distinct paged needs, layers in each, for every run the (group, layer) or None of each of its needs,
+    the (run, index among the run's needs) of every per-request need)."""
     group_needs: List[Any] = []
     layers_in_group: List[int] = []
-    layer_of_run: List[Optional[Tuple[int, int]]] = []
-    per_request: List[int] = []
+    layer_of_run: List[List[Optional[Tuple[int, int]]]] = []
+    per_request: List[Tuple[int, int]] = []
     for i, (need, cache_of) in enumerate(needs):
-        paged = need is not None and cache_kind(need).paged
-        if not paged:
+        subs = _flat(need)
+        if cache_of is not None and len(subs) != 1:
+            raise ValueError(f"run {i} reads the cache of run {cache_of} but its mixer keeps " +
+                             ("no paged cache" if not subs else "several caches"))
+        placed: List[Optional[Tuple[int, int]]] = []
+        for j, sub in enumerate(subs):
+            if not cache_kind(sub).paged:
+                if cache_of is not None:
+                    raise ValueError(f"run {i} reads the cache of run {cache_of} but its mixer keeps no paged cache")
+                placed.append(None)
+                per_request.append((i, j))
+                continue
             if cache_of is not None:
-                raise ValueError(f"run {i} reads the cache of run {cache_of} but its mixer keeps no paged cache")
-            layer_of_run.append(None)
-            if need is not None:
-                per_request.append(i)
-            continue
-        if cache_of is not None:
-            src_need = needs[cache_of][0]
-            if src_need != need or layer_of_run[cache_of] is None:
-                raise ValueError(f"run {i} reads the cache of run {cache_of}, whose cache has other sizes: {src_need} vs {need}")
-            layer_of_run.append(layer_of_run[cache_of])
-            continue
-        if need not in group_needs:
-            group_needs.append(need)
-            layers_in_group.append(0)
-        g = group_needs.index(need)
-        layer_of_run.append((g, layers_in_group[g]))
-        layers_in_group[g] += 1
+                src = _flat(needs[cache_of][0])
+                if len(src) != 1 or src[0] != sub or layer_of_run[cache_of][0] is None:
+                    raise ValueError(f"run {i} reads the cache of run {cache_of}, whose cache has other sizes: {needs[cache_of][0]} vs {sub}")
+                placed.append(layer_of_run[cache_of][0])
+                continue
+            if sub not in group_needs:
+                group_needs.append(sub)
+                layers_in_group.append(0)
+            g = group_needs.index(sub)
+            placed.append((g, layers_in_group[g]))
+            layers_in_group[g] += 1
+        layer_of_run.append(placed)
     return group_needs, layers_in_group, layer_of_run, per_request
 
 
@@ -83,18 +96,22 @@ class CacheManager:
         self.views: List[CacheView] = []
         self._per_request: List[Tuple[CacheKind, Any, Any]] = []      # (kind, need, storage) of the runs with such needs
         for i, (need, cache_of) in enumerate(needs):
-            if need is None:
-                self.views.append(CacheView("none"))
-            elif layer_of_run[i] is not None:
-                g, layer = layer_of_run[i]
-                grp = self.groups[g]
-                self.views.append(grp.kind.page_view(grp.storage, need, layer, g, page_size, grp.num_pages, cache_of is None))
+            views = []
+            for sub, placed in zip(_flat(need), layer_of_run[i]):
+                if placed is not None:
+                    g, layer = placed
+                    grp = self.groups[g]
+                    views.append(grp.kind.page_view(grp.storage, sub, layer, g, page_size, grp.num_pages, cache_of is None))
+                else:
+                    kind = cache_kind(sub)
+                    storage = kind.allocate_slots(sub, max_requests, device)
+                    self._per_request.append((kind, sub, storage))
+                    views.append(kind.slot_view(storage, sub))
+            if isinstance(need, tuple):     # a mixer made of several: a part for each of its needs, in their order
+                self.views.append(CacheView("several", parts=tuple(views)))
             else:
-                kind = cache_kind(need)
-                storage = kind.allocate_slots(need, max_requests, device)
-                self._per_request.append((kind, need, storage))
-                self.views.append(kind.slot_view(storage, need))
-        self.core = HostCore([(page_size, g.num_pages, g.kind.window(g.need)) for g in self.groups], max_requests,
+                self.views.append(views[0] if views else CacheView("none"))
+        self.core = HostCore([(page_size, g.num_pages, g.kind.window(g.need), g.kind.keep_first(g.need)) for g in self.groups], max_requests,
                              token_budget, max_chunk, max_positions)
 
     @staticmethod
@@ -108,7 +125,7 @@ class CacheManager:
         group_needs, layers_in_group, _, per_request = _group_runs(needs)
         if not group_needs:
             return []
-        fixed = sum(cache_kind(needs[i][0]).bytes_per_request(needs[i][0]) for i in per_request) * max_requests
+        fixed = sum(cache_kind(sub).bytes_per_request(sub) for sub in (_flat(needs[i][0])[j] for i, j in per_request)) * max_requests
         budget = int(max(free_bytes - fixed, 0) * fraction)
         step = min(max_step_tokens or max_seq_len, max_seq_len)
         caps, costs = [], []
@@ -117,7 +134,7 @@ class CacheManager:
             held = max_seq_len
             if kind.window(need) > 0:
                 # a page's worth more than the span: the span starts anywhere in a page
-                held = min(held, kind.window(need) + step + page_size)
+                held = min(held, kind.window(need) + step + page_size + -(-kind.keep_first(need) // page_size) * page_size)
             caps.append(max_requests * -(-held // page_size))
             costs.append(n_layers * kind.bytes_per_token(need, dtype) * page_size)
         lo, hi = 1, max(caps)          # the most pages P with sum(cost * min(cap, P)) within the budget, at least one

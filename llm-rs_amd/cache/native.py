@@ -23,7 +23,7 @@ def _lib():
     lib = load_host()
     if not _configured:
         lib.llmrs_core_create.restype = c_void_p
-        lib.llmrs_core_create.argtypes = [c_int, POINTER(c_int), POINTER(c_int), POINTER(c_int), c_int, c_int, c_int, c_int]
+        lib.llmrs_core_create.argtypes = [c_int, POINTER(c_int), POINTER(c_int), POINTER(c_int), POINTER(c_int), c_int, c_int, c_int, c_int]
         lib.llmrs_core_destroy.argtypes = [c_void_p]
         lib.llmrs_core_error.restype = c_char_p
         lib.llmrs_core_error.argtypes = [c_void_p]
@@ -85,14 +85,16 @@ class BatchOffsets:
 
 
 class HostCore:
-    """One cache manager + scheduler.  `groups` is a list of (page_size, num_pages, window)."""
+    """One cache manager + scheduler.  `groups` is a list of (page_size, num_pages, window) or
+    (page_size, num_pages, window, keep_first): with a window, the first keep_first positions of a request stay
+    visible for good, and their pages are never given back."""
 
     def __init__(self, groups: Sequence[Sequence[int]], max_requests: int, token_budget: int = 2048,
                  max_chunk: int = 0, max_positions: int = 1 << 30):
         self._lib = _lib()
         n = len(groups)
-        arr = lambda i: (c_int * max(n, 1))(*[int(g[i]) for g in groups])
-        self._h = self._lib.llmrs_core_create(n, arr(0), arr(1), arr(2), max_requests, token_budget, max_chunk, max_positions)
+        arr = lambda i: (c_int * max(n, 1))(*[int(g[i]) if i < len(g) else 0 for g in groups])
+        self._h = self._lib.llmrs_core_create(n, arr(0), arr(1), arr(2), arr(3), max_requests, token_budget, max_chunk, max_positions)
         if not self._h:
             raise CoreError(self._lib.llmrs_create_error().decode())
         self.n_groups = n

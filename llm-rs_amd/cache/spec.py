@@ -2,7 +2,7 @@
 kind of need becomes memory.
 
 A need is a small frozen value (`PagedKV`, `FixedState`, or one of a class that somebody
-registered); the `CacheKind` registered for its class says what it costs and how it is laid out.
+registered), or a tuple of such values for a mixer made of several (it gets a view with a part for each); the `CacheKind` registered for its class says what it costs and how it is laid out.
 There are two families.  A *paged* kind holds something for every token of a request: runs
 of the schedule with equal needs share a pool of pages and one block table per request, and a
 window lets pages that no later query can see go back.  A *per-request* kind holds something
@@ -21,11 +21,13 @@ import torch
 class PagedKV:
     """Keys and values in pages; `window` > 0 means only that many of the latest
     keys stay visible, so older pages can go back to the pool.  `value_dim`: the width of a
-    value when it is not the width of a key (0: the same)."""
+    value when it is not the width of a key (0: the same).  `keep_first`: with a window, the
+    first so many positions of a request stay visible too, and their pages stay."""
     kv_heads: int
     head_dim: int
     window: int = 0
     value_dim: int = 0
+    keep_first: int = 0
 
     @property
     def v_dim(self) -> int:
@@ -42,7 +44,7 @@ class FixedState:
 @dataclass
 class CacheView:
     """What one run's mixer sees of the cache."""
-    kind: str                       # "paged", "state", "none", or what another kind calls itself
+    kind: str                       # "paged", "state", "none", "several", or what another kind calls itself
     group: int = -1                 # index into the step's slot maps and block tables (paged kinds)
     k: Optional[torch.Tensor] = None
     v: Optional[torch.Tensor] = None
@@ -51,6 +53,7 @@ class CacheView:
     writes: bool = True
     state: Optional[torch.Tensor] = None   # [max_requests, *shape]
     data: Any = None                # whatever a kind registered from outside hands its mixer
+    parts: Tuple["CacheView", ...] = ()    # kind "several": a view for each need of a mixer that asked for several
 
 
 class CacheKind:
@@ -61,6 +64,10 @@ class CacheKind:
     # -- paged kinds ---------------------------------------------------------------
     def window(self, need) -> int:
         """Tokens that stay visible (0: all): pages that lie wholly before them go back to the pool."""
+        return 0
+
+    def keep_first(self, need) -> int:
+        """With a window: the first so many positions stay visible for good (their pages are never given back)."""
         return 0
 
     def bytes_per_token(self, need, dtype: torch.dtype) -> int:
@@ -97,6 +104,9 @@ class _PagedKVKind(CacheKind):
 
     def window(self, need):
         return need.window
+
+    def keep_first(self, need):
+        return need.keep_first if need.window > 0 else 0
 
     def bytes_per_token(self, need, dtype):
         return need.kv_heads * (need.head_dim + need.v_dim) * dtype.itemsize

@@ -8,6 +8,7 @@ import os
 from typing import Any, Callable, Dict
 
 from .llama import ConfigError, LlamaConfig
+from .lilatar import LilatarConfig
 from .tuvodra import TuvodraConfig
 
 # name -> function(config dict) -> typed config with .model_spec() and .to_dict()
@@ -35,7 +36,9 @@ def config_from_dict(d: Dict[str, Any]):
 
 
 def load_config(path: str):
-    """`path` is a model folder or its config.json."""
+    """`path` is a model folder or its config.json.  An architecture some of whose sizes only the tensors' shapes
+    give (`sizes_from_tensors`) is shown the shapes of the folder's tensors, read from the files' headers."""
+    folder = path if os.path.isdir(path) else os.path.dirname(path)
     if os.path.isdir(path):
         path = os.path.join(path, "config.json")
     try:
@@ -43,8 +46,17 @@ def load_config(path: str):
             d = json.load(f)
     except FileNotFoundError:
         raise ConfigError(f"no config.json at {path}") from None
-    return config_from_dict(d)
+    config = config_from_dict(d)
+    if hasattr(config, "sizes_from_tensors"):
+        from ..weights.loader import open_model_files
+        from ..weights.safetensors_io import SafetensorsError
+        try:
+            config.sizes_from_tensors({name: tuple(f.entries[name][1]) for name, f in open_model_files(folder).items()})
+        except (SafetensorsError, OSError):
+            pass            # no tensors beside the configuration: the sizes must be in the file
+    return config
 
 
 register_architecture("LlamaForCausalLM", LlamaConfig.from_dict)
 register_architecture("Tuvodra", TuvodraConfig.from_dict)
+register_architecture("Lilatar", LilatarConfig.from_dict)

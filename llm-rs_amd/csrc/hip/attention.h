@@ -13,9 +13,24 @@ struct AttnArgs {
     // dist_r1[head] * ln(1 + dist_r2[head] * (i - j)), in 32-bit.  Both null: none.
     const float* dist_r1;
     const float* dist_r2;
+    // > 0: the scaled score s becomes softcap * tanh(s / softcap), in 32-bit, before any penalty and the softmax.
+    float softcap;
+    // With a window: the first keep_first positions of a request stay visible to every later query, at their true
+    // positions.  Key j is visible to the query at i when j <= i and (i - j < window or j < keep_first).
+    int keep_first;
 };
-// Whether a call is the plain one (values as wide as keys, no distance penalty) that every kernel file takes.
-static inline bool attn_is_plain(const AttnArgs& a) { return a.v_dim == a.head_dim && a.dist_r1 == nullptr; }
+// Whether a call is the plain one (values as wide as keys, no distance penalty, no soft cap, no kept first keys) that
+// every kernel file takes.
+static inline bool attn_is_plain(const AttnArgs& a) {
+    return a.v_dim == a.head_dim && a.dist_r1 == nullptr && a.softcap <= 0.0f && (a.keep_first <= 0 || a.window <= 0);
+}
+// The first key of the window of the query at `pos`, and how many of the first keys lie before it and stay visible.
+__host__ __device__ static inline int attn_window_lo(const AttnArgs& a, int pos) {
+    return (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+}
+__host__ __device__ static inline int attn_kept_before(const AttnArgs& a, int lo) {
+    return a.keep_first < lo ? (a.keep_first > 0 ? a.keep_first : 0) : lo;
+}
 
 #if defined(__HIPCC__)
 // A step's entries bring their tokens as tiles of `per` tokens that never cross an entry; entries with one token

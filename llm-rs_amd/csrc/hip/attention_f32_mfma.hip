@@ -41,7 +41,11 @@ __device__ __forceinline__ void f32_walk(const f32x4 (&qf)[HD / 8], const float*
                                          const int* __restrict__ table, const AttnArgs& a, int kvh, int c, int h, int pos, int lo,
                                          int t_begin, int t_end, f32x16 (&O)[HD / 32], float& m, float& l) {
     const int ps = a.page_size;
-    const float scale_log2e = a.scale * 1.44269504088896341f;     // exponentials in base 2: one multiply-add and one v_exp_f32
+    const float log2e = 1.44269504088896341f;
+    const float scale_log2e = a.scale * log2e;                    // exponentials in base 2: one multiply-add and one v_exp_f32
+    const bool capped = a.softcap > 0.0f;                         // scores bent into (-cap, cap) first
+    const float inv_cap = capped ? 1.0f / a.softcap : 0.0f, cap_log2e = a.softcap * log2e;
+    const int keep = a.keep_first;                                // first keys that stay visible when the window has passed them
     auto page_of = [&](int key) {
         int pg = table[min(key / ps, a.table_width - 1)];
         return min(max(pg, 0), a.num_pages - 1);                   // stay inside the cache whatever the table holds
@@ -82,7 +86,8 @@ __device__ __forceinline__ void f32_walk(const f32x4 (&qf)[HD / 8], const float*
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             int kk = t0 + 8 * (i >> 2) + 4 * h + (i & 3);
-            S[i] = (kk > pos || kk < lo) ? -INFINITY : S[i] * scale_log2e;
+            float sc = capped ? cap_log2e * tanhf(S[i] * a.scale * inv_cap) : S[i] * scale_log2e;
+            S[i] = (kk > pos || (kk < lo && kk >= keep)) ? -INFINITY : sc;
             mx = fmaxf(mx, S[i]);
         }
         mx = fmaxf(mx, swap_halves(mx));
@@ -153,6 +158,9 @@ __global__ __launch_bounds__(256) void attn_f32_tiles_kernel(const float* __rest
 #pragma unroll
         for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
     float m = -INFINITY, l = 0.0f;
+    // the first keys that stay visible, where they lie before the tiles of the window (those among the window's tiles
+    // pass the mask there)
+    if (a.keep_first > 0 && t_begin > 0) f32_walk<HD>(qf, kc, vc, table, a, kvh, c, h, pos, lo, 0, min(a.keep_first, t_begin), O, m, l);
     f32_walk<HD>(qf, kc, vc, table, a, kvh, c, h, pos, lo, t_begin, t_end, O, m, l);
     if (!cvalid) return;
     float inv = 1.0f / l;
@@ -202,6 +210,8 @@ __global__ __launch_bounds__(64) void attn_f32_split_kernel(const float* __restr
 #pragma unroll
         for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
     float m = -INFINITY, l = 0.0f;
+    if (ch == 0 && a.keep_first > 0 && (begin & ~31) > 0)      // the first chunk's wave also takes the kept first keys
+        f32_walk<HD>(qf, kc, vc, table, a, kvh, c, h, pos, lo, 0, min(a.keep_first, begin & ~31), O, m, l);
     f32_walk<HD>(qf, kc, vc, table, a, kvh, c, h, pos, lo, begin & ~31, end, O, m, l);
     if (!cvalid) return;
     float* pp = partial + ((size_t)(e * a.n_heads + head) * max_chunks + ch) * (HD + 2);
@@ -224,7 +234,7 @@ int llmrs_attention_f32_mfma(hipStream_t stream, const float* q, float* out, con
                              const int* block_table, const int* positions, const int* q_starts, int n_entries,
                              int skip_single, const AttnArgs& a) {
     int G = a.n_heads / a.n_kv_heads;
-    if (!attn_is_plain(a)) return 0;
+    if (a.v_dim != a.head_dim || a.dist_r1 != nullptr) return 0;
     if (a.head_dim % 32 || a.head_dim > 256 || a.page_size % 4 || G > 32 || q_starts == nullptr) return 0;
     if (a.q_stride % 4 || a.out_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)out & 15) || ((uintptr_t)k_cache & 15) ||
         ((uintptr_t)v_cache & 15))
@@ -253,7 +263,7 @@ int llmrs_attention_f32_mfma_split(hipStream_t stream, const float* q, float* pa
                                    const int* block_table, const int* q_starts, const int* seq_lens, int n_entries,
                                    int max_chunks, const AttnArgs& a) {
     int G = a.n_heads / a.n_kv_heads;
-    if (!attn_is_plain(a)) return 0;
+    if (a.v_dim != a.head_dim || a.dist_r1 != nullptr) return 0;
     if (a.head_dim % 32 || a.head_dim > 256 || a.page_size % 4 || G > 32 || q_starts == nullptr || seq_lens == nullptr) return 0;
     if (a.q_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) || ((uintptr_t)v_cache & 15) || ((uintptr_t)partial & 7))
         return 0;

@@ -3,7 +3,8 @@
 //
 // For the query at position p of its request, head h, kv head g = h / (heads per
 // kv head): keys j = lo..p with lo = 0 or p + 1 - window; s_j = (q . k_j) * scale;
-// softmax over j, computed online with a running maximum, all in 32-bit;
+// (optionally bent into (-cap, cap) by cap * tanh(s / cap), and with a window optionally also the first few keys
+// of the request, walked before the window's); softmax over j, computed online with a running maximum, all in 32-bit;
 // o = sum_j softmax_j v_j, divided by the sum at the end.  The mask is the loop's
 // bound.  This is the reference's paged_attention (shaders/ops.metal:636-758;
 // causal_len of :673-674 equals p + 1) with a tile of 64 keys, one per lane.
@@ -55,6 +56,7 @@ __device__ __forceinline__ void walk_keys(const float* qs, const T* __restrict__
                 for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], to_f32(kp[d]), dot);
             }
             s = dot * a.scale;
+            if (a.softcap > 0.0f) s = a.softcap * tanhf(s / a.softcap);
             if (far) s -= r1 * logf(fmaf(r2, (float)(pos - j), 1.0f));
         }
         float m_new = fmaxf(m, wave_max(s));
@@ -99,6 +101,8 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
     float m = -INFINITY, l = 0.0f;
     float acc[MAX_HEAD_DIM / 64] = {};
+    int kept = attn_kept_before(a, lo);         // first keys that the window has passed and that stay visible
+    if (kept > 0) walk_keys<T, VEC>(qs, k_cache, v_cache, table, a, kvh, h, pos, 0, kept, m, l, acc);
     walk_keys<T, VEC>(qs, k_cache, v_cache, table, a, kvh, h, pos, lo, pos + 1, m, l, acc);
     T* orow = out + (size_t)t * a.out_stride + (size_t)h * a.v_dim;
 #pragma unroll
@@ -132,6 +136,8 @@ __global__ __launch_bounds__(64) void attention_generic_split_kernel(
     __syncthreads();
     float m = -INFINITY, l = 0.0f;
     float acc[MAX_HEAD_DIM / 64] = {};
+    int kept = ch == 0 ? attn_kept_before(a, lo) : 0;      // the first chunk's wave also takes the kept first keys
+    if (kept > 0) walk_keys<T, VEC>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, h, pos, 0, kept, m, l, acc);
     walk_keys<T, VEC>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, h, pos, begin, end, m, l, acc);
     float* pp = partial + ((size_t)(e * a.n_heads + h) * max_chunks + ch) * (a.v_dim + 2);
     if (lane == 0) { pp[0] = m; pp[1] = l; }
@@ -193,6 +199,7 @@ __device__ __forceinline__ void walk_keys_group(const float* qs, const T* __rest
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 s[g] = dot[g] * a.scale;
+                if (a.softcap > 0.0f) s[g] = a.softcap * tanhf(s[g] / a.softcap);
                 if (far) s[g] -= r1[g] * logf(fmaf(r2[g], (float)(pos - j), 1.0f));
             }
         }
@@ -249,6 +256,8 @@ __global__ __launch_bounds__(64) void attention_generic_group_tokens_kernel(
 #pragma unroll
         for (int i = 0; i < NACC; ++i) acc[g][i] = 0.0f;
     }
+    int kept = attn_kept_before(a, lo);
+    if (kept > 0) walk_keys_group<T, VEC, G>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, pos, 0, kept, m, l, acc);
     walk_keys_group<T, VEC, G>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, pos, lo, pos + 1, m, l, acc);
 #pragma unroll
     for (int g = 0; g < G; ++g) {
@@ -288,6 +297,8 @@ __global__ __launch_bounds__(64) void attention_generic_group_kernel(
 #pragma unroll
         for (int i = 0; i < NACC; ++i) acc[g][i] = 0.0f;
     }
+    int kept = ch == 0 ? attn_kept_before(a, lo) : 0;
+    if (kept > 0) walk_keys_group<T, VEC, G>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, pos, 0, kept, m, l, acc);
     walk_keys_group<T, VEC, G>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, pos, begin, end, m, l, acc);
 #pragma unroll
     for (int g = 0; g < G; ++g) {
@@ -463,13 +474,15 @@ static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cac
 // the matrix-core kernels choose the keys per wave by it.
 // v_dim: the width of a value (the cache's values are [page][kv_head][v_dim][slot], `out` has v_dim per head);
 // dist_r1, dist_r2: [n_heads] 32-bit, the logarithmic distance penalty of AttnArgs, or both null.
+// softcap, keep_first: the soft cap of the scores and the first keys that a window keeps (AttnArgs), or 0.
 extern "C" int llmrs_attention_ext(hipStream_t stream, int dtype, const void* q, int q_stride, void* out, int out_stride,
                                    const void* k_cache, const void* v_cache, const int* block_table, int table_width,
                                    const int* token_entry, const int* positions, const int* q_starts,
                                    const int* seq_lens, int n_entries, int n_tokens, int n_heads, int n_kv_heads,
                                    int head_dim, int page_size, int num_pages, int window, float scale,
                                    void* scratch, size_t scratch_bytes, int max_seq_len, int n_single, long single_keys,
-                                   int allow_mfma, int v_dim, const float* dist_r1, const float* dist_r2) {
+                                   int allow_mfma, int v_dim, const float* dist_r1, const float* dist_r2, float softcap,
+                                   int keep_first) {
     LLMRS_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && v_dim > 0, "attention: bad sizes");
     LLMRS_REQUIRE(v_dim <= MAX_HEAD_DIM, "attention: value width %d exceeds %d", v_dim, MAX_HEAD_DIM);
     LLMRS_REQUIRE((dist_r1 == nullptr) == (dist_r2 == nullptr), "attention: the distance penalty needs both of its tables");
@@ -478,13 +491,14 @@ extern "C" int llmrs_attention_ext(hipStream_t stream, int dtype, const void* q,
     LLMRS_REQUIRE(page_size > 0 && table_width > 0 && num_pages > 0, "attention: bad cache geometry");
     LLMRS_REQUIRE(q_stride >= n_heads * head_dim && out_stride >= n_heads * v_dim, "attention: row stride too short");
     LLMRS_REQUIRE(window >= 0, "attention: negative window");
+    LLMRS_REQUIRE(softcap >= 0.0f && keep_first >= 0, "attention: negative soft cap or number of kept first keys");
     LLMRS_REQUIRE(n_heads <= 65535, "attention: too many heads for one launch");
     LLMRS_REQUIRE(n_single <= n_entries, "attention: %d single-token entries among %d entries", n_single, n_entries);
     LLMRS_REQUIRE(n_single != n_entries || n_tokens == n_entries,
                   "attention: every entry is said to bring one token, but %d entries bring %d tokens", n_entries, n_tokens);
     if (n_tokens == 0) return 0;
     AttnArgs a{n_tokens, n_heads, n_kv_heads, head_dim, page_size, table_width, num_pages, q_stride, out_stride, window, scale,
-               v_dim, dist_r1, dist_r2};
+               v_dim, dist_r1, dist_r2, softcap, window > 0 ? keep_first : 0};
     if (dtype == LLMRS_BF16 && allow_mfma) {
         int took = llmrs_attention_bf16_mfma(stream, (const bf16*)q, (bf16*)out, (const bf16*)k_cache, (const bf16*)v_cache,
                                              block_table, token_entry, positions, q_starts, seq_lens, n_entries,
@@ -517,5 +531,5 @@ extern "C" int llmrs_attention(hipStream_t stream, int dtype, const void* q, int
     return llmrs_attention_ext(stream, dtype, q, q_stride, out, out_stride, k_cache, v_cache, block_table, table_width,
                                token_entry, positions, q_starts, seq_lens, n_entries, n_tokens, n_heads, n_kv_heads,
                                head_dim, page_size, num_pages, window, scale, scratch, scratch_bytes, max_seq_len, n_single,
-                               single_keys, allow_mfma, head_dim, nullptr, nullptr);
+                               single_keys, allow_mfma, head_dim, nullptr, nullptr, 0.0f, 0);
 }

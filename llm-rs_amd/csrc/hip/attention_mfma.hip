@@ -1149,6 +1149,7 @@ int llmrs_attention_bf16_mfma(hipStream_t stream, const bf16* q, bf16* out, cons
     (void)token_entry;
     int G = a.n_heads / a.n_kv_heads;
     if (a.v_dim != a.head_dim) return 0;               // (a distance penalty is these kernels' too)
+    if (a.softcap > 0.0f || a.keep_first > 0) return 0;   // soft-capped scores and kept first keys: the caller's other kernels
     if (a.page_size != 16 || a.head_dim % 32 || G > 32 || q_starts == nullptr) return 0;
     if (a.q_stride % 8 || a.out_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)out & 7)) return 0;
     if (n_entries > 65535 || a.n_kv_heads > 65535) return 0;

@@ -1,0 +1,319 @@
+// Mixers whose memory is a matrix per head, S [key channel][value channel], carried from token to token in 32-bit:
+//
+//   S <- decay * S                      decay: one number per head, or one per (token, head, key channel)
+//   u  = beta (v - S^T k)               with a write strength beta per (token, head): the delta rule;
+//   u  = v                              without: plain linear attention
+//   S <- S + k u^T;    o = S^T q        (the read-out sees the current token's write)
+//
+// and what stands around them: the activation of q, k and v where a projection leaves them raw, unit norms of q and k
+// with the decay and the write strength of a gated delta rule, the RMS norm of the read-out under a sigmoid gate.
+// Every column of S (one value channel) evolves by itself, so the columns are shared out over lanes; a column's rows
+// are shared out over LANES_PER_COLUMN lanes that add their partial dot products up by cross-lane moves.  A step's
+// entries (prompt portions and single tokens alike) each start from their request's state and leave it.
+#include "common.h"
+
+#define LANES_PER_COLUMN 8
+#define SCAN_THREADS 256
+#define COLUMNS_PER_BLOCK (SCAN_THREADS / LANES_PER_COLUMN)
+
+struct LinearScanArgs {
+    const float* q; int ldq;            // [T, qk_heads * dk]
+    const float* k; int ldk;            // [T, qk_heads * dk]
+    const float* v; int ldv;            // [T, heads * dv]
+    const float* g; int ldg;            // [T, heads * dk] decay per key channel, or null
+    const float* decay;                 // [heads] decay per head, or null (both null: none)
+    const float* beta; int ldb;         // [T, heads] write strength of the delta rule, or null: plain linear attention
+    float* state; long state_stride;    // [slots][heads][dk][dv]
+    float* out; int ldo;                // [T, heads * dv]
+    int heads, qk_heads, dk, dv;
+};
+
+__device__ __forceinline__ float column_sum(float x) {
+#pragma unroll
+    for (int d = 1; d < LANES_PER_COLUMN; d <<= 1) x += __shfl_xor(x, d, 64);
+    return x;
+}
+
+// R: rows of a column that one lane holds (rows part * R .. part * R + R - 1; those past dk are idle).
+// VEC: dk % 4 == 0 and all row strides and bases allow 16-byte loads of four consecutive rows.
+template <int R, bool VEC, bool DELTA, bool CHANNEL_DECAY>
+__global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(const int* __restrict__ q_starts, const int* __restrict__ slots,
+                                                                    LinearScanArgs a) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int part = lane & (LANES_PER_COLUMN - 1);
+    const int col = blockIdx.x * COLUMNS_PER_BLOCK + wave * (64 / LANES_PER_COLUMN) + (lane >> 3);
+    const int h = blockIdx.y, e = blockIdx.z;
+    const int kh = h / (a.heads / a.qk_heads);
+    const bool live = col < a.dv;
+    const int j = live ? col : a.dv - 1;
+    const int r0 = part * R;
+    const int t0 = q_starts[e], t1 = q_starts[e + 1];
+    if (t0 >= t1) return;
+    float* sp = a.state + (size_t)slots[e] * a.state_stride + (size_t)h * a.dk * a.dv + j;
+    float s[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) s[i] = (r0 + i < a.dk) ? sp[(size_t)(r0 + i) * a.dv] : 0.0f;
+    const float head_decay = (!CHANNEL_DECAY && a.decay) ? a.decay[h] : 1.0f;
+
+    float kc[R], qc[R], gc[CHANNEL_DECAY ? R : 1];
+    float vc = 0.0f, bc = 1.0f;
+    auto fetch = [&](int t, float (&kk)[R], float (&qq)[R], float (&gg)[CHANNEL_DECAY ? R : 1], float& vv, float& bb) {
+        const float* kp = a.k + (size_t)t * a.ldk + (size_t)kh * a.dk + r0;
+        const float* qp = a.q + (size_t)t * a.ldq + (size_t)kh * a.dk + r0;
+        const float* gp = CHANNEL_DECAY ? a.g + (size_t)t * a.ldg + (size_t)h * a.dk + r0 : nullptr;
+        if constexpr (VEC) {
+#pragma unroll
+            for (int i = 0; i < R; i += 4) {
+                bool in = r0 + i < a.dk;          // (dk % 4 == 0: four rows are in or out together)
+                float4 x = in ? *(const float4*)(kp + i) : make_float4(0, 0, 0, 0);
+                float4 y = in ? *(const float4*)(qp + i) : make_float4(0, 0, 0, 0);
+                kk[i] = x.x; kk[i + 1] = x.y; kk[i + 2] = x.z; kk[i + 3] = x.w;
+                qq[i] = y.x; qq[i + 1] = y.y; qq[i + 2] = y.z; qq[i + 3] = y.w;
+                if constexpr (CHANNEL_DECAY) {
+                    float4 z = in ? *(const float4*)(gp + i) : make_float4(1, 1, 1, 1);
+                    gg[i] = z.x; gg[i + 1] = z.y; gg[i + 2] = z.z; gg[i + 3] = z.w;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                bool in = r0 + i < a.dk;
+                kk[i] = in ? kp[i] : 0.0f;
+                qq[i] = in ? qp[i] : 0.0f;
+                if constexpr (CHANNEL_DECAY) gg[i] = in ? gp[i] : 1.0f;
+            }
+        }
+        vv = a.v[(size_t)t * a.ldv + (size_t)h * a.dv + j];
+        bb = DELTA ? a.beta[(size_t)t * a.ldb + h] : 1.0f;
+    };
+    fetch(t0, kc, qc, gc, vc, bc);
+    for (int t = t0; t < t1; ++t) {
+        float kn[R], qn[R], gn[CHANNEL_DECAY ? R : 1];
+        float vn = 0.0f, bn = 1.0f;
+        if (t + 1 < t1) fetch(t + 1, kn, qn, gn, vn, bn);          // the next token's operands travel while this one is folded in
+        float u = vc;
+        if constexpr (DELTA) {
+            float d0 = 0.0f, d1 = 0.0f;
+#pragma unroll
+            for (int i = 0; i < R; i += 2) {
+                s[i] *= CHANNEL_DECAY ? gc[i] : head_decay;
+                s[i + 1] *= CHANNEL_DECAY ? gc[i + 1] : head_decay;
+                d0 = fmaf(kc[i], s[i], d0);
+                d1 = fmaf(kc[i + 1], s[i + 1], d1);
+            }
+            u = bc * (vc - column_sum(d0 + d1));
+        } else {
+#pragma unroll
+            for (int i = 0; i < R; ++i) s[i] *= CHANNEL_DECAY ? gc[i] : head_decay;
+        }
+        float o0 = 0.0f, o1 = 0.0f;
+#pragma unroll
+        for (int i = 0; i < R; i += 2) {
+            s[i] = fmaf(kc[i], u, s[i]);
+            s[i + 1] = fmaf(kc[i + 1], u, s[i + 1]);
+            o0 = fmaf(qc[i], s[i], o0);
+            o1 = fmaf(qc[i + 1], s[i + 1], o1);
+        }
+        float o = column_sum(o0 + o1);
+        if (live && part == 0) a.out[(size_t)t * a.ldo + (size_t)h * a.dv + j] = o;
+        if (t + 1 < t1) {
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                kc[i] = kn[i]; qc[i] = qn[i];
+                if constexpr (CHANNEL_DECAY) gc[i] = gn[i];
+            }
+            vc = vn; bc = bn;
+        }
+    }
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+            if (r0 + i < a.dk) sp[(size_t)(r0 + i) * a.dv] = s[i];
+    }
+}
+
+static bool entries_given(const int* q_starts, const int* slots, int n_entries) { return q_starts && slots && n_entries > 0 && n_entries <= 65535; }
+
+// q, k: [T, qk_heads * dk]; v: [T, heads * dv]; g: [T, heads * dk] or null; decay: [heads] or null; beta: [T, heads] or
+// null (no delta correction); state: [slots][heads * dk * dv] at state_stride floats a slot, read at an entry's first
+// token and left at its last; out: [T, heads * dv].  All 32-bit.  Head h reads the q and k of head h / (heads / qk_heads).
+extern "C" int llmrs_linear_scan(hipStream_t stream, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
+                                 const float* g, int ldg, const float* decay, const float* beta, int ldb, float* state,
+                                 long state_stride, const int* q_starts, const int* slots, int n_entries, int n_tokens,
+                                 int heads, int qk_heads, int dk, int dv, float* out, int ldo) {
+    LLMRS_REQUIRE(heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && dk > 0 && dv > 0, "linear_scan: bad sizes");
+    LLMRS_REQUIRE(dk <= 32 * LANES_PER_COLUMN, "linear_scan: %d key channels exceed %d", dk, 32 * LANES_PER_COLUMN);
+    LLMRS_REQUIRE(ldq >= qk_heads * dk && ldk >= qk_heads * dk && ldv >= heads * dv && ldo >= heads * dv, "linear_scan: row stride too short");
+    LLMRS_REQUIRE(!g || ldg >= heads * dk, "linear_scan: the decays' rows are too short");
+    LLMRS_REQUIRE(!(g && decay), "linear_scan: a decay per head or per channel, not both");
+    LLMRS_REQUIRE(!beta || ldb >= heads, "linear_scan: the write strengths' rows are too short");
+    LLMRS_REQUIRE(state_stride >= (long)heads * dk * dv && heads <= 65535, "linear_scan: the state does not fit its slot");
+    LLMRS_REQUIRE(entries_given(q_starts, slots, n_entries), "linear_scan: bad entries");
+    if (n_tokens == 0) return 0;
+    LinearScanArgs a{q, ldq, k, ldk, v, ldv, g, ldg, decay, beta, ldb, state, state_stride, out, ldo, heads, qk_heads, dk, dv};
+    int per_lane = ceil_div(dk, LANES_PER_COLUMN);
+    int R = per_lane <= 4 ? 4 : per_lane <= 8 ? 8 : per_lane <= 16 ? 16 : 32;
+    auto aligned = [](const void* p, int ld) { return ((uintptr_t)p & 15) == 0 && ld % 4 == 0; };
+    bool vec = dk % 4 == 0 && aligned(q, ldq) && aligned(k, ldk) && (!g || aligned(g, ldg));
+    dim3 grid(ceil_div(dv, COLUMNS_PER_BLOCK), heads, n_entries);
+#define SCAN(RR, V, D, C) linear_scan_kernel<RR, V, D, C><<<grid, SCAN_THREADS, 0, stream>>>(q_starts, slots, a)
+#define BY_ROWS(V, D, C) do { if (R == 4) SCAN(4, V, D, C); else if (R == 8) SCAN(8, V, D, C); else if (R == 16) SCAN(16, V, D, C); else SCAN(32, V, D, C); } while (0)
+#define BY_KIND(V) do { if (beta && g) BY_ROWS(V, true, true); else if (beta) BY_ROWS(V, true, false); else if (g) BY_ROWS(V, false, true); else BY_ROWS(V, false, false); } while (0)
+    if (vec) BY_KIND(true); else BY_KIND(false);
+#undef BY_KIND
+#undef BY_ROWS
+#undef SCAN
+    LLMRS_LAUNCH_CHECK("linear_scan");
+    return 0;
+}
+
+// ---- x <- silu(x) on the columns [col0, col0 + n) of 32-bit rows --------------------------------------------------
+__global__ void silu_columns_kernel(float* __restrict__ x, int ld, int col0, int n, long total) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    long t = i / n;
+    int c = (int)(i - t * n);
+    float* p = x + (size_t)t * ld + col0 + c;
+    *p = silu_f32(*p);
+}
+
+extern "C" int llmrs_silu_columns(hipStream_t stream, float* x, int ld, int n_rows, int col0, int n) {
+    LLMRS_REQUIRE(x && ld >= col0 + n && col0 >= 0 && n > 0 && n_rows >= 0, "silu_columns: bad sizes");
+    long total = (long)n_rows * n;
+    if (total == 0) return 0;
+    LLMRS_REQUIRE(ceil_div(total, 256) <= 0x7fffffff, "silu_columns: too many elements for one launch");
+    silu_columns_kernel<<<ceil_div(total, 256), 256, 0, stream>>>(x, ld, col0, n, total);
+    LLMRS_LAUNCH_CHECK("silu_columns");
+    return 0;
+}
+
+// ---- what a gated delta rule needs between its convolutions and its recurrence ------------------------------------
+// In place, all 32-bit.  One wave for each (token, unit), the units being the q heads, the k heads and the heads:
+//   q head: x <- x / sqrt(sum(x^2) + unit_eps) * dk^(-1/2)          k head: x <- x / sqrt(sum(x^2) + unit_eps)
+//   head h: a[t, h, :] <- exp(-exp(A_log[h]) * softplus(a[t, h, :] + dt_bias[h, :])),  b[t, h] <- sigmoid(b[t, h])
+__device__ __forceinline__ float softplus_f32(float x) { return x > 20.0f ? x : log1pf(expf(x)); }
+
+__global__ __launch_bounds__(64) void delta_prepare_kernel(float* __restrict__ q, int ldq, float* __restrict__ k, int ldk,
+                                                            float* __restrict__ a, int lda, float* __restrict__ b, int ldb,
+                                                            const float* __restrict__ A_log, const float* __restrict__ dt_bias,
+                                                            int heads, int qk_heads, int dk, float unit_eps) {
+    int t = blockIdx.x, unit = blockIdx.y, lane = threadIdx.x;
+    if (unit < 2 * qk_heads) {
+        bool is_q = unit < qk_heads;
+        float* row = is_q ? q + (size_t)t * ldq + (size_t)unit * dk : k + (size_t)t * ldk + (size_t)(unit - qk_heads) * dk;
+        float ss = 0.0f;
+        for (int d = lane; d < dk; d += 64) ss = fmaf(row[d], row[d], ss);
+        float inv = 1.0f / sqrtf(wave_sum(ss) + unit_eps);
+        if (is_q) inv *= 1.0f / sqrtf((float)dk);
+        for (int d = lane; d < dk; d += 64) row[d] *= inv;
+        return;
+    }
+    int h = unit - 2 * qk_heads;
+    float rate = expf(A_log[h]);
+    float* row = a + (size_t)t * lda + (size_t)h * dk;
+    for (int d = lane; d < dk; d += 64) row[d] = expf(-rate * softplus_f32(row[d] + dt_bias[(size_t)h * dk + d]));
+    if (lane == 0) {
+        float* bp = b + (size_t)t * ldb + h;
+        *bp = 1.0f / (1.0f + expf(-*bp));
+    }
+}
+
+extern "C" int llmrs_delta_prepare(hipStream_t stream, float* q, int ldq, float* k, int ldk, float* a, int lda, float* b, int ldb,
+                                   const float* A_log, const float* dt_bias, int n_tokens, int heads, int qk_heads, int dk,
+                                   float unit_eps) {
+    LLMRS_REQUIRE(q && k && a && b && A_log && dt_bias && heads > 0 && qk_heads > 0 && dk > 0 && n_tokens >= 0, "delta_prepare: bad arguments");
+    LLMRS_REQUIRE(ldq >= qk_heads * dk && ldk >= qk_heads * dk && lda >= heads * dk && ldb >= heads, "delta_prepare: row stride too short");
+    LLMRS_REQUIRE(heads + 2 * qk_heads <= 65535, "delta_prepare: too many heads for one launch");
+    if (n_tokens == 0) return 0;
+    delta_prepare_kernel<<<dim3(n_tokens, heads + 2 * qk_heads), 64, 0, stream>>>(q, ldq, k, ldk, a, lda, b, ldb, A_log, dt_bias,
+                                                                                 heads, qk_heads, dk, unit_eps);
+    LLMRS_LAUNCH_CHECK("delta_prepare");
+    return 0;
+}
+
+// ---- RMS norm in groups under a sigmoid gate ------------------------------------------------------------------------
+// out[t, c] = x[t, c] / sqrt(mean over c's group of x^2 + eps) * weight[c % weight_len] * sigmoid(gate[t, c]);
+// groups of `group` consecutive columns; x and gate 32-bit, out in the activation type.  One block a (token, group).
+template <class T>
+__global__ __launch_bounds__(256) void gated_rmsnorm_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ gate, int ldg,
+                                                             const float* __restrict__ weight, int weight_len, int group, float eps,
+                                                             T* __restrict__ out, int ldo) {
+    __shared__ float partial[4];
+    int t = blockIdx.x, c0 = blockIdx.y * group, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float* xr = x + (size_t)t * ldx + c0;
+    float ss = 0.0f;
+    for (int d = threadIdx.x; d < group; d += 256) ss = fmaf(xr[d], xr[d], ss);
+    ss = wave_sum(ss);
+    if (lane == 0) partial[wave] = ss;
+    __syncthreads();
+    float inv = 1.0f / sqrtf((partial[0] + partial[1] + partial[2] + partial[3]) / (float)group + eps);
+    const float* gr = gate + (size_t)t * ldg + c0;
+    T* orow = out + (size_t)t * ldo + c0;
+    for (int d = threadIdx.x; d < group; d += 256) {
+        float sig = 1.0f / (1.0f + expf(-gr[d]));
+        orow[d] = from_f32<T>(xr[d] * inv * weight[(c0 + d) % weight_len] * sig);
+    }
+}
+
+extern "C" int llmrs_gated_rmsnorm(hipStream_t stream, int dtype, const float* x, int ldx, const float* gate, int ldg,
+                                   const float* weight, int weight_len, int n_tokens, int n_groups, int group, float eps,
+                                   void* out, int ldo) {
+    LLMRS_REQUIRE(x && gate && weight && out && n_groups > 0 && group > 0 && weight_len > 0, "gated_rmsnorm: bad arguments");
+    long width = (long)n_groups * group;
+    LLMRS_REQUIRE(ldx >= width && ldg >= width && ldo >= width && n_groups <= 65535, "gated_rmsnorm: row stride too short");
+    LLMRS_REQUIRE(weight_len == group || weight_len == width, "gated_rmsnorm: a weight per column of the row or of a group");
+    if (n_tokens == 0) return 0;
+    dim3 grid(n_tokens, n_groups);
+    if (dtype == LLMRS_F32)
+        gated_rmsnorm_kernel<float><<<grid, 256, 0, stream>>>(x, ldx, gate, ldg, weight, weight_len, group, eps, (float*)out, ldo);
+    else if (dtype == LLMRS_BF16)
+        gated_rmsnorm_kernel<bf16><<<grid, 256, 0, stream>>>(x, ldx, gate, ldg, weight, weight_len, group, eps, (bf16*)out, ldo);
+    else
+        return llmrs_fail("gated_rmsnorm: unknown dtype %d", dtype);
+    LLMRS_LAUNCH_CHECK("gated_rmsnorm");
+    return 0;
+}
+
+// ---- sums of normed rows added into the stream ---------------------------------------------------------------------
+// out[t, :] += coef * sum_i rmsnorm(x_i[t, :] + bias_i) * w_i,   i < n_in (1 or 2), all 32-bit, rows of D.
+// The norm after a sublayer (n_in = 1, coef = 1), and the mean of two mixers' normed outputs (n_in = 2, coef = 1/2).
+__global__ __launch_bounds__(256) void rmsnorm_sum_kernel(float* __restrict__ out, const float* __restrict__ x0, const float* __restrict__ b0,
+                                                           const float* __restrict__ w0, const float* __restrict__ x1,
+                                                           const float* __restrict__ b1, const float* __restrict__ w1, int D,
+                                                           float coef, float eps) {
+    __shared__ float partial[2][4];
+    int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float* r0 = x0 + (size_t)t * D;
+    const float* r1 = x1 ? x1 + (size_t)t * D : nullptr;
+    float s0 = 0.0f, s1 = 0.0f;
+    for (int d = threadIdx.x; d < D; d += 256) {
+        float a = r0[d] + (b0 ? b0[d] : 0.0f);
+        s0 = fmaf(a, a, s0);
+        if (r1) {
+            float b = r1[d] + (b1 ? b1[d] : 0.0f);
+            s1 = fmaf(b, b, s1);
+        }
+    }
+    s0 = wave_sum(s0);
+    s1 = wave_sum(s1);
+    if (lane == 0) { partial[0][wave] = s0; partial[1][wave] = s1; }
+    __syncthreads();
+    float inv0 = 1.0f / sqrtf((partial[0][0] + partial[0][1] + partial[0][2] + partial[0][3]) / (float)D + eps);
+    float inv1 = 1.0f / sqrtf((partial[1][0] + partial[1][1] + partial[1][2] + partial[1][3]) / (float)D + eps);
+    float* orow = out + (size_t)t * D;
+    for (int d = threadIdx.x; d < D; d += 256) {
+        float y = (r0[d] + (b0 ? b0[d] : 0.0f)) * inv0 * w0[d];
+        if (r1) y += (r1[d] + (b1 ? b1[d] : 0.0f)) * inv1 * w1[d];
+        orow[d] += coef * y;
+    }
+}
+
+extern "C" int llmrs_rmsnorm_sum(hipStream_t stream, float* out, const float* x0, const float* b0, const float* w0, const float* x1,
+                                 const float* b1, const float* w1, int n_rows, int D, float coef, float eps) {
+    LLMRS_REQUIRE(out && x0 && w0 && D > 0 && n_rows >= 0, "rmsnorm_sum: bad arguments");
+    LLMRS_REQUIRE((x1 == nullptr) == (w1 == nullptr) && (x1 || !b1), "rmsnorm_sum: the second input needs rows and a weight");
+    if (n_rows == 0) return 0;
+    rmsnorm_sum_kernel<<<n_rows, 256, 0, stream>>>(out, x0, b0, w0, x1, b1, w1, D, coef, eps);
+    LLMRS_LAUNCH_CHECK("rmsnorm_sum");
+    return 0;
+}

@@ -1,8 +1,9 @@
-// What lies between a q/k/v projection and attention for mixers that neither rotate nor leave q and k as they come:
-// biases, a norm of q and k to unit root mean square per head, and the write of k and v into the paged cache, in one
-// pass over the projection's 32-bit sums.
+// What lies between a q/k/v projection and attention for mixers that do more to q and k than rotate them:
+// biases, a norm of q and k to unit root mean square per head, a rotation by position, and the write of k and v into
+// the paged cache, in one pass over the projection's 32-bit sums.
 //
-//   q[t, h, :] = unit(sums_q[t, h, :] + bias_q[h, :])      unit(x) = x / sqrt(mean(x^2) + eps) over the head (eps 0: x)
+//   q[t, h, :] = rot(unit(sums_q[t, h, :] + bias_q[h, :]))   unit(x) = x / sqrt(mean(x^2) + eps) over the head (eps 0: x)
+//   rot: features (2i, 2i + 1), i < rotary_dim / 2, turned by the angle position * inv_freq[i]; the others pass
 //   k likewise, into its page; v[t, g, :] = sums_v + bias_v, into its page (values lie transposed, cache_layout.h).
 // Everything is computed in 32-bit and rounded once to the activation type on the way out.
 #include "cache_layout.h"
@@ -13,13 +14,16 @@ struct QkvFinishArgs {
     int in_stride, q_stride;       // elements between tokens in the sums and in q
     int page_size, num_pages, write_kv;
     float eps;                     // of the unit norm; 0: q and k are not normed
+    int rotary_dim;                // 0: no rotation
 };
 
 // One wave for each (token, head of q, k or v).
 template <class T>
 __global__ __launch_bounds__(64) void qkv_finish_kernel(const float* __restrict__ sums, const float* __restrict__ bias,
                                                          T* __restrict__ q, const int* __restrict__ slot_map,
-                                                         T* __restrict__ k_cache, T* __restrict__ v_cache, QkvFinishArgs a) {
+                                                         T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                                         const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                                         QkvFinishArgs a) {
     int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     bool is_q = head < a.n_heads, is_k = !is_q && head < a.n_heads + a.n_kv_heads;
     if (!is_q && !a.write_kv) return;
@@ -38,6 +42,22 @@ __global__ __launch_bounds__(64) void qkv_finish_kernel(const float* __restrict_
     }
     float inv = 1.0f;
     if ((is_q || is_k) && a.eps > 0.0f) inv = 1.0f / sqrtf(wave_sum(ss) / (float)width + a.eps);
+    if ((is_q || is_k) && a.rotary_dim > 0) {
+        // feature d's partner d ^ 1 lies in the neighbouring lane; angles and the turn in 32-bit
+        float pos = (float)positions[t];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int d = lane + 64 * i;
+            x[i] *= inv;
+            float other = __shfl_xor(x[i], 1, 64);
+            if (d < a.rotary_dim) {
+                float s, c;
+                sincosf(pos * inv_freq[d >> 1], &s, &c);
+                x[i] = (d & 1) ? fmaf(x[i], c, other * s) : fmaf(x[i], c, -other * s);
+            }
+        }
+        inv = 1.0f;
+    }
     if (is_q) {
         T* dst = q + (size_t)t * a.q_stride + col;
 #pragma unroll
@@ -64,23 +84,27 @@ __global__ __launch_bounds__(64) void qkv_finish_kernel(const float* __restrict_
 // sums: [n_tokens, in_stride] 32-bit, a token's q heads, then its k heads, then its v heads; bias: the same columns
 // (or null); q: [n_tokens, q_stride] in `dtype`; the caches in `dtype`; slot_map: [n_tokens] page * page_size + slot.
 // n_kv_heads 0: the projection has no k and v (a mixer that reads another's cache).
+// positions: [n_tokens], inv_freq: [rotary_dim / 2] 32-bit, for the rotation (rotary_dim 0: none).
 extern "C" int llmrs_qkv_finish(hipStream_t stream, int dtype, const float* sums, int in_stride, const float* bias, void* q,
                                 int q_stride, const int* slot_map, void* k_cache, void* v_cache, int n_tokens, int n_heads,
-                                int n_kv_heads, int head_dim, int v_dim, int page_size, int num_pages, int write_kv, float eps) {
+                                int n_kv_heads, int head_dim, int v_dim, int page_size, int num_pages, int write_kv, float eps,
+                                const int* positions, const float* inv_freq, int rotary_dim) {
     LLMRS_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0 && v_dim > 0, "qkv_finish: bad sizes");
     LLMRS_REQUIRE(head_dim <= 512 && v_dim <= 512, "qkv_finish: heads of %d / %d features exceed 512", head_dim, v_dim);
     LLMRS_REQUIRE(in_stride >= (n_heads + n_kv_heads) * head_dim + n_kv_heads * v_dim && q_stride >= n_heads * head_dim,
                   "qkv_finish: row stride too short");
     LLMRS_REQUIRE(eps >= 0.0f, "qkv_finish: negative eps");
+    LLMRS_REQUIRE(rotary_dim >= 0 && rotary_dim % 2 == 0 && rotary_dim <= head_dim, "qkv_finish: a rotation of %d features does not fit heads of %d", rotary_dim, head_dim);
+    LLMRS_REQUIRE(rotary_dim == 0 || (positions && inv_freq), "qkv_finish: a rotation needs positions and frequencies");
     LLMRS_REQUIRE(!write_kv || (page_size > 0 && num_pages > 0 && slot_map && k_cache && v_cache), "qkv_finish: no cache to write");
     LLMRS_REQUIRE(n_heads + 2 * n_kv_heads <= 65535, "qkv_finish: too many heads for one launch");
     if (n_tokens == 0) return 0;
-    QkvFinishArgs a{n_tokens, n_heads, n_kv_heads, head_dim, v_dim, in_stride, q_stride, page_size, num_pages, write_kv, eps};
+    QkvFinishArgs a{n_tokens, n_heads, n_kv_heads, head_dim, v_dim, in_stride, q_stride, page_size, num_pages, write_kv, eps, rotary_dim};
     dim3 grid(n_tokens, n_heads + 2 * n_kv_heads);
     if (dtype == LLMRS_F32)
-        qkv_finish_kernel<float><<<grid, 64, 0, stream>>>(sums, bias, (float*)q, slot_map, (float*)k_cache, (float*)v_cache, a);
+        qkv_finish_kernel<float><<<grid, 64, 0, stream>>>(sums, bias, (float*)q, slot_map, (float*)k_cache, (float*)v_cache, positions, inv_freq, a);
     else if (dtype == LLMRS_BF16)
-        qkv_finish_kernel<bf16><<<grid, 64, 0, stream>>>(sums, bias, (bf16*)q, slot_map, (bf16*)k_cache, (bf16*)v_cache, a);
+        qkv_finish_kernel<bf16><<<grid, 64, 0, stream>>>(sums, bias, (bf16*)q, slot_map, (bf16*)k_cache, (bf16*)v_cache, positions, inv_freq, a);
     else
         return llmrs_fail("qkv_finish: unknown dtype %d", dtype);
     LLMRS_LAUNCH_CHECK("qkv_finish");

@@ -73,3 +73,22 @@ extern "C" int llmrs_scale_softcap_rows(hipStream_t stream, float* logits, int l
     LLMRS_LAUNCH_CHECK("scale_softcap_rows");
     return 0;
 }
+
+// rows[t, c] += bias[c], in 32-bit: the bias of a projection whose product was added into 32-bit rows.
+__global__ void add_bias_rows_kernel(float* __restrict__ rows, int ld, const float* __restrict__ bias, int n, long total) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    long t = i / n;
+    int c = (int)(i - t * n);
+    rows[(size_t)t * ld + c] += bias[c];
+}
+
+extern "C" int llmrs_add_bias_rows(hipStream_t stream, float* rows, int ld, const float* bias, int n_rows, int n) {
+    LLMRS_REQUIRE(rows && bias && n > 0 && ld >= n && n_rows >= 0, "add_bias_rows: bad arguments");
+    long total = (long)n_rows * n;
+    if (total == 0) return 0;
+    LLMRS_REQUIRE((total + 255) / 256 <= 0x7fffffffL, "add_bias_rows: too many elements for one launch");
+    add_bias_rows_kernel<<<(int)((total + 255) / 256), 256, 0, stream>>>(rows, ld, bias, n, total);
+    LLMRS_LAUNCH_CHECK("add_bias_rows");
+    return 0;
+}

@@ -72,11 +72,11 @@ extern "C" {
 
 const char* llmrs_create_error() { return g_create_error.c_str(); }
 
-void* llmrs_core_create(int n_groups, const int* page_size, const int* num_pages, const int* window,
+void* llmrs_core_create(int n_groups, const int* page_size, const int* num_pages, const int* window, const int* keep_first,
                         int max_requests, int token_budget, int max_chunk, int max_positions) {
     try {
         std::vector<GroupSpec> groups;
-        for (int g = 0; g < n_groups; ++g) groups.push_back({page_size[g], num_pages[g], window[g]});
+        for (int g = 0; g < n_groups; ++g) groups.push_back({page_size[g], num_pages[g], window[g], keep_first ? keep_first[g] : 0});
         auto core = std::make_unique<Core>();
         core->cache = std::make_unique<CacheManager>(groups, max_requests);
         core->scheduler = std::make_unique<Scheduler>(*core->cache, token_budget, max_chunk, max_positions);

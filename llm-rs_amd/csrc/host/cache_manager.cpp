@@ -1,5 +1,6 @@
 #include "cache_manager.h"
 
+#include <algorithm>
 #include <stdexcept>
 
 namespace llmrs {
@@ -11,6 +12,7 @@ CacheManager::CacheManager(const std::vector<GroupSpec>& groups, int max_request
         if (g.page_size <= 0) throw std::invalid_argument("page_size must be positive");
         if (g.num_pages <= 0) throw std::invalid_argument("num_pages must be positive");
         if (g.window < 0) throw std::invalid_argument("window must not be negative");
+        if (g.keep_first < 0) throw std::invalid_argument("keep_first must not be negative");
         pools_.emplace_back(g.num_pages);
     }
     for (int s = max_requests - 1; s >= 0; --s) free_slots_.push_back(s);
@@ -58,7 +60,7 @@ void CacheManager::drop_passed(int slot, int g, int start) {
     int keep_from = first_visible(g, start) / ps;  // first logical page still visible
     auto& t = tables_[slot][g];
     for (int i = 0; i < keep_from && i < (int)t.size(); ++i) {
-        if (t[i] >= 0) {
+        if (t[i] >= 0 && !page_wanted(g, i, start)) {
             pools_[g].give_back(t[i]);
             t[i] = -1;
         }
@@ -69,7 +71,8 @@ int CacheManager::pages_needed(int g, int start, int count) const {
     int ps = groups_[g].page_size;
     int first = first_visible(g, start) / ps;
     int last = (start + count + ps - 1) / ps;
-    return last - first;
+    int kept = std::min((groups_[g].keep_first + ps - 1) / ps, first);     // pages of the first positions, below the window
+    return last - first + kept;
 }
 
 bool CacheManager::ensure(int slot, int start, int count) {
@@ -81,20 +84,18 @@ bool CacheManager::ensure(int slot, int start, int count) {
     for (int g = 0; g < num_groups(); ++g) {
         int ps = groups_[g].page_size;
         int need = (start + count + ps - 1) / ps - (int)tables_[slot][g].size();
-        // Logical pages below the visible range are never taken, so a request that
+        // Logical pages that no query from `start` on can see are never taken, so a request that
         // starts late in a window group (after a recompute) holds holes there.
-        int first = first_visible(g, start) / ps;
         int have = (int)tables_[slot][g].size();
         int fresh = 0;
-        for (int i = have; i < have + (need > 0 ? need : 0); ++i) fresh += i >= first;
+        for (int i = have; i < have + (need > 0 ? need : 0); ++i) fresh += page_wanted(g, i, start);
         if (fresh > pools_[g].available()) return false;
     }
     for (int g = 0; g < num_groups(); ++g) {
         int ps = groups_[g].page_size;
         int last = (start + count + ps - 1) / ps;
-        int first = first_visible(g, start) / ps;
         auto& t = tables_[slot][g];
-        while ((int)t.size() < last) t.push_back((int)t.size() >= first ? pools_[g].take() : -1);
+        while ((int)t.size() < last) t.push_back(page_wanted(g, (int)t.size(), start) ? pools_[g].take() : -1);
     }
     return true;
 }

@@ -6,7 +6,8 @@
 // holds positions [i*page_size, (i+1)*page_size), or -1 once a window has passed
 // it and the page went back to the pool.  A group with window w keeps only the
 // pages that a query at the request's next position can still see (keys at
-// positions > p - w); a group with window 0 keeps all.
+// positions > p - w, and the first keep_first positions where the group keeps
+// those for good); a group with window 0 keeps all.
 //
 // Reference: PagedKVPool + ensure_blocks (src/kv_pool.rs:12-95) is the single
 // group, all-keys case; RequestTable (src/serve/engine.rs:69-92) is the stable
@@ -24,6 +25,9 @@ struct GroupSpec {
     int page_size;
     int num_pages;
     int window;  // 0: every key stays visible
+    // With a window: the first `keep_first` positions of a request stay visible to every later
+    // query whatever the window has passed, so the pages that hold them are never given back.
+    int keep_first = 0;
 };
 
 class CacheManager {
@@ -58,6 +62,11 @@ public:
     int first_visible(int g, int pos) const {
         int w = groups_[g].window;
         return (w <= 0 || pos + 1 <= w) ? 0 : pos + 1 - w;
+    }
+    // Whether logical page `page` holds a position that a query at `pos` or later can see.
+    bool page_wanted(int g, int page, int pos) const {
+        int ps = groups_[g].page_size;
+        return page >= first_visible(g, pos) / ps || (long long)page * ps < groups_[g].keep_first;
     }
 
 private:

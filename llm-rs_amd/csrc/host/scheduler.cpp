@@ -34,7 +34,8 @@ void Scheduler::check(int n_prompt, int max_new) const {
         if (w > 0) {
             int n = std::min({max_chunk_, budget_, computed});
             long long span = std::min<long long>((long long)w + n - 1, computed);
-            worst = std::min<long long>(worst, span <= 1 ? 1 : (span - 1 + ps - 1) / ps + 1);
+            int kept = (cache_.group(g).keep_first + ps - 1) / ps;      // pages of first positions that are never given back
+            worst = std::min<long long>(worst, (span <= 1 ? 1 : (span - 1 + ps - 1) / ps + 1) + kept);
         }
         if (worst > cache_.pages_total(g))
             throw std::invalid_argument("request needs " + std::to_string(worst) + " pages of cache group " +

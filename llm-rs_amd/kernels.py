@@ -188,11 +188,19 @@ class HipKernels(Kernels):
             "llmrs_argmax_rows": [V, V, I, I, I, V, V, c_size_t],
             "llmrs_sample_rows": [V, V, I, I, I, V, V],
             "llmrs_place_ids": [V, V, I, V, V, V, I, I, I],
-            "llmrs_attention_ext": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, ctypes.c_long, I, I, V, V],
+            "llmrs_attention_ext": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, ctypes.c_long, I, I, V, V, F, I],
             "llmrs_group_rmsnorm": [V, I, V, V, ctypes.c_long, I, V, V, V, I, I, I, F, V, V, V, V, V],
             "llmrs_streams_mix": [V, V, ctypes.c_long, I, V, V, V, ctypes.c_long],
             "llmrs_streams_copy_first": [V, V, ctypes.c_long, I, ctypes.c_long],
-            "llmrs_qkv_finish": [V, I, V, I, V, V, I, V, V, V, I, I, I, I, I, I, I, I, F],
+            "llmrs_qkv_finish": [V, I, V, I, V, V, I, V, V, V, I, I, I, I, I, I, I, I, F, V, V, I],
+            "llmrs_linear_scan": [V, V, I, V, I, V, I, V, I, V, V, I, V, ctypes.c_long, V, V, I, I, I, I, I, I, V, I],
+            "llmrs_silu_columns": [V, V, I, I, I, I],
+            "llmrs_delta_prepare": [V, V, I, V, I, V, I, V, I, V, V, I, I, I, I, F],
+            "llmrs_gated_rmsnorm": [V, I, V, I, V, I, V, I, I, I, I, F, V, I],
+            "llmrs_rmsnorm_sum": [V, V, V, V, V, V, V, V, I, I, F, F],
+            "llmrs_route_topk": [V, V, I, V, I, I, I, I, I],
+            "llmrs_act_weight": [V, I, V, I, V, I, I, I, I, I, V, I],
+            "llmrs_add_bias_rows": [V, V, I, V, I, I],
             "llmrs_mingru_scan": [V, I, V, I, V, V, V, ctypes.c_long, V, V, I, I, V, I, I, V],
             "llmrs_causal_conv_silu": [V, I, V, I, V, V, V, ctypes.c_long, V, V, V, I, I, I, I, V, I],
             "llmrs_selective_scan": [V, I, V, I, V, I, I, I, V, I, V, V, V, V, I, V, ctypes.c_long, V, V, V, I, I, I, I, V, I, I, V],
@@ -406,18 +414,20 @@ class HipKernels(Kernels):
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
                   n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1,
-                  single_keys=0, value_dim=0, distance=None) -> None:
+                  single_keys=0, value_dim=0, distance=None, softcap=0.0, keep_first=0) -> None:
         """single_keys: how many keys the single-token entries see together (windows counted), 0 if unknown.
         value_dim: the width of a value where it is not a key's (0: the same).  distance: (r1, r2), float32 [n_heads]
-        each: r1[h] * ln(1 + r2[h] * (i - j)) is taken off the scaled score of query i and key j."""
+        each: r1[h] * ln(1 + r2[h] * (i - j)) is taken off the scaled score of query i and key j.  softcap > 0: the
+        scaled score s becomes softcap * tanh(s / softcap).  keep_first: with a window, the request's first so many
+        keys stay visible to every later query."""
         assert q.stride(1) == 1 and out.stride(1) == 1 and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype
         assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
         v_dim = int(value_dim) or head_dim
         assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim and v_cache.numel() == num_pages * n_kv_heads * page_size * v_dim
-        if v_dim != head_dim or distance is not None:
+        if v_dim != head_dim or distance is not None or softcap > 0 or (keep_first > 0 and window > 0):
             return self._attention_ext(q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens, n_heads,
                                        n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch, max_seq_len, n_single,
-                                       single_keys, v_dim, distance)
+                                       single_keys, v_dim, distance, softcap, keep_first)
         T = q.shape[0]
         assert token_entry.shape[0] == T and positions.shape[0] == T and out.shape[0] == T
         moved = flops = 0
@@ -436,7 +446,7 @@ class HipKernels(Kernels):
 
     def _attention_ext(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens, n_heads,
                        n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch, max_seq_len, n_single, single_keys,
-                       v_dim, distance) -> None:
+                       v_dim, distance, softcap=0.0, keep_first=0) -> None:
         T = q.shape[0]
         assert token_entry.shape[0] == T and positions.shape[0] == T and out.shape[0] == T
         r1 = r2 = None
@@ -446,7 +456,7 @@ class HipKernels(Kernels):
         moved = flops = 0
         if self.times is not None:
             keys = int(seq_lens.sum().item())
-            seen = int((positions + 1).sum().item()) if window <= 0 else int((positions + 1).clamp(max=window).sum().item())
+            seen = int((positions + 1).sum().item()) if window <= 0 else int((positions + 1).clamp(max=window + keep_first).sum().item())
             moved = (keys * n_kv_heads * (head_dim + v_dim) + T * n_heads * (head_dim + v_dim)) * q.element_size()
             flops = 2 * seen * n_heads * (head_dim + v_dim)
         self._run(f"attention {T} tokens" + (" (decode)" if n_single == block_table.shape[0] else ""), moved, flops, q.dtype,
@@ -455,7 +465,7 @@ class HipKernels(Kernels):
                   _p(block_table), block_table.shape[1], _p(token_entry), _p(positions), _p(q_starts), _p(seq_lens),
                   block_table.shape[0], T, n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale,
                   _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size(), int(max_seq_len),
-                  int(n_single), int(single_keys), int(self.allow_mfma), v_dim, _p(r1), _p(r2))
+                  int(n_single), int(single_keys), int(self.allow_mfma), v_dim, _p(r1), _p(r2), float(softcap), int(keep_first))
 
     # out[i, :] = weight * groupnorm(sum_s w_in[s] * x[s][rows[i] or i, :]); x: [T, D] or [S, T, D] float32
     def group_rmsnorm(self, out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, groups: int,
@@ -501,9 +511,13 @@ class HipKernels(Kernels):
 
     def qkv_finish(self, sums: torch.Tensor, bias: Optional[torch.Tensor], q: torch.Tensor, slot_map, k_cache, v_cache,
                    n_heads: int, n_kv_heads: int, head_dim: int, v_dim: int, page_size: int, num_pages: int, write_kv: bool,
-                   eps: float) -> None:
+                   eps: float, positions: Optional[torch.Tensor] = None, inv_freq: Optional[torch.Tensor] = None, rotary_dim: int = 0) -> None:
         """sums [T, q | k | v] float32 -> q [T, heads * head_dim] (activation type) and the cache's pages: biases
-        added, q and k divided by their root mean square over the head (eps > 0), one rounding on the way out."""
+        added, q and k divided by their root mean square over the head (eps > 0), then (rotary_dim > 0) their features
+        (2i, 2i + 1) turned by positions[t] * inv_freq[i]; one rounding on the way out."""
+        if rotary_dim:
+            assert positions.dtype == torch.int32 and positions.shape[0] == sums.shape[0] and inv_freq.dtype == torch.float32
+            assert inv_freq.shape[0] == rotary_dim // 2 and inv_freq.is_contiguous() and rotary_dim % 2 == 0 and rotary_dim <= head_dim
         assert sums.dtype == torch.float32 and sums.stride(1) == 1 and q.stride(1) == 1 and q.shape[0] == sums.shape[0]
         width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * v_dim
         assert sums.shape[1] == width and (bias is None or (bias.dtype == torch.float32 and bias.numel() == width and bias.is_contiguous()))
@@ -514,7 +528,98 @@ class HipKernels(Kernels):
         T = sums.shape[0]
         self._run("qkv_finish", T * width * (4 + q.element_size()), 4 * T * width, None, self.lib.llmrs_qkv_finish,
                   self._stream(), _code(q.dtype), _p(sums), sums.stride(0), _p(bias), _p(q), q.stride(0), _p(slot_map),
-                  _p(k_cache), _p(v_cache), T, n_heads, n_kv_heads, head_dim, v_dim, page_size, num_pages, int(write_kv), float(eps))
+                  _p(k_cache), _p(v_cache), T, n_heads, n_kv_heads, head_dim, v_dim, page_size, num_pages, int(write_kv), float(eps),
+                  _p(positions) if rotary_dim else None, _p(inv_freq) if rotary_dim else None, int(rotary_dim))
+
+    def add_bias_rows(self, rows: torch.Tensor, bias: torch.Tensor) -> None:
+        """rows[t, :] += bias; both float32."""
+        assert rows.dtype == bias.dtype == torch.float32 and rows.stride(1) == 1 and bias.numel() == rows.shape[1] and bias.is_contiguous()
+        self._run(f"add_bias {rows.shape[0]}x{rows.shape[1]}", rows.numel() * 8, rows.numel(), None,
+                  self.lib.llmrs_add_bias_rows, self._stream(), _p(rows), rows.stride(0), _p(bias), rows.shape[0], rows.shape[1])
+
+    def linear_scan(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, q_starts, slots, heads: int,
+                    qk_heads: int, dk: int, dv: int, out: torch.Tensor, decay: Optional[torch.Tensor] = None,
+                    g: Optional[torch.Tensor] = None, beta: Optional[torch.Tensor] = None) -> None:
+        """Per head a matrix S [dk, dv] carried from token to token: S <- decay S (decay [heads], or g [T, heads * dk] a
+        key channel); u = beta (v - S^T k) (beta [T, heads]; None: u = v); S <- S + k u^T; out = S^T q.  q, k
+        [T, qk_heads * dk], v and out [T, heads * dv], all float32 with unit column stride; state [slots, >= heads * dk * dv]
+        float32, read at an entry's first token and left at its last."""
+        T = q.shape[0]
+        for t in (q, k, v, out, g, beta):
+            assert t is None or (t.dtype == torch.float32 and t.stride(1) == 1 and t.shape[0] == T)
+        assert q.shape[1] == k.shape[1] == qk_heads * dk and v.shape[1] == out.shape[1] == heads * dv
+        assert state.dtype == torch.float32 and state.stride(-1) == 1 and state.shape[1] >= heads * dk * dv
+        assert q_starts.dtype == slots.dtype == torch.int32 and q_starts.numel() == slots.numel() + 1
+        assert decay is None or (decay.dtype == torch.float32 and decay.numel() == heads and decay.is_contiguous())
+        assert g is None or g.shape[1] == heads * dk
+        assert beta is None or beta.shape[1] == heads
+        kind = ("delta" if beta is not None else "decay") + (" by channel" if g is not None else "")
+        self._run(f"linear_scan {T}x{heads}x{dk}x{dv} {kind}", T * (2 * qk_heads * dk + (heads * dk if g is not None else 0) + 2 * heads * dv) * 4
+                  + slots.numel() * heads * dk * dv * 8, (7 if beta is not None else 5) * T * heads * dk * dv, None,
+                  self.lib.llmrs_linear_scan, self._stream(), _p(q), q.stride(0), _p(k), k.stride(0), _p(v), v.stride(0),
+                  _p(g), 0 if g is None else g.stride(0), _p(decay), _p(beta), 0 if beta is None else beta.stride(0),
+                  _p(state), state.stride(0), _p(q_starts), _p(slots), slots.numel(), T, heads, qk_heads, dk, dv, _p(out), out.stride(0))
+
+    def silu_columns(self, x: torch.Tensor, col0: int, n: int) -> None:
+        """x[:, col0:col0 + n] <- silu of itself; x float32 with unit column stride."""
+        assert x.dtype == torch.float32 and x.stride(1) == 1 and 0 <= col0 and col0 + n <= x.shape[1]
+        self._run(f"silu {x.shape[0]}x{n}", x.shape[0] * n * 8, 4 * x.shape[0] * n, None,
+                  self.lib.llmrs_silu_columns, self._stream(), _p(x), x.stride(0), x.shape[0], int(col0), int(n))
+
+    def delta_prepare(self, q: torch.Tensor, k: torch.Tensor, a: torch.Tensor, b: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor,
+                      heads: int, qk_heads: int, dk: int, unit_eps: float) -> None:
+        """In place, float32: q, k [T, qk_heads * dk] made unit vectors per head (x / sqrt(sum x^2 + unit_eps)), q also
+        times dk^(-1/2); a [T, heads * dk] <- exp(-exp(A_log[h]) softplus(a + dt_bias)); b [T, heads] <- sigmoid(b)."""
+        T = q.shape[0]
+        for t in (q, k, a, b):
+            assert t.dtype == torch.float32 and t.stride(1) == 1 and t.shape[0] == T
+        assert q.shape[1] == k.shape[1] == qk_heads * dk and a.shape[1] == heads * dk and b.shape[1] == heads
+        assert A_log.dtype == dt_bias.dtype == torch.float32 and A_log.numel() == heads and dt_bias.numel() == heads * dk
+        assert A_log.is_contiguous() and dt_bias.is_contiguous()
+        self._run(f"delta_prepare {T}x{heads}x{dk}", T * (2 * qk_heads + heads) * dk * 8, 8 * T * (2 * qk_heads + heads) * dk, None,
+                  self.lib.llmrs_delta_prepare, self._stream(), _p(q), q.stride(0), _p(k), k.stride(0), _p(a), a.stride(0),
+                  _p(b), b.stride(0), _p(A_log), _p(dt_bias), T, heads, qk_heads, dk, float(unit_eps))
+
+    def gated_rmsnorm(self, out: torch.Tensor, x: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, group: int, eps: float) -> None:
+        """out[t, c] = x[t, c] / sqrt(mean of x^2 over c's group of `group` columns + eps) * weight[c % len(weight)] *
+        sigmoid(gate[t, c]); x, gate float32, weight float32 of a group's or a row's length."""
+        T, W = x.shape
+        assert x.dtype == gate.dtype == weight.dtype == torch.float32 and x.stride(1) == gate.stride(1) == out.stride(1) == 1
+        assert gate.shape == x.shape and out.shape == x.shape and W % group == 0 and weight.numel() in (group, W) and weight.is_contiguous()
+        self._run(f"gated_rmsnorm {T}x{W}", T * W * (8 + out.element_size()), 8 * T * W, None,
+                  self.lib.llmrs_gated_rmsnorm, self._stream(), _code(out.dtype), _p(x), x.stride(0), _p(gate), gate.stride(0),
+                  _p(weight), weight.numel(), T, W // group, int(group), float(eps), _p(out), out.stride(0))
+
+    def rmsnorm_sum(self, out: torch.Tensor, inputs, coef: float, eps: float) -> None:
+        """out += coef * sum of rmsnorm(x + bias) * weight over `inputs`, one or two (x [T, D], bias [D] or None,
+        weight [D]); everything float32 and contiguous."""
+        assert 1 <= len(inputs) <= 2 and out.dtype == torch.float32 and out.is_contiguous()
+        T, D = out.shape
+        flat = []
+        for x, bias, weight in inputs:
+            assert x.dtype == weight.dtype == torch.float32 and x.is_contiguous() and tuple(x.shape) == (T, D) and weight.numel() == D
+            assert bias is None or (bias.dtype == torch.float32 and bias.numel() == D)
+            flat += [_p(x), _p(bias), _p(weight)]
+        flat += [None] * (6 - len(flat))
+        self._run(f"rmsnorm_sum {T}x{D} of {len(inputs)}", T * D * 4 * (2 + len(inputs)), 6 * len(inputs) * T * D, None,
+                  self.lib.llmrs_rmsnorm_sum, self._stream(), _p(out), *flat, T, D, float(coef), float(eps))
+
+    def route_topk(self, logits: torch.Tensor, weights: torch.Tensor, top: int, renormalize: bool = False) -> None:
+        """weights[t, e] = softmax(logits[t])[e] for the `top` experts with the largest scores (of equal ones the lower
+        index), 0 for the others; with `renormalize` divided by the chosen scores' sum.  Both float32 [T, experts]."""
+        assert logits.dtype == weights.dtype == torch.float32 and logits.stride(1) == weights.stride(1) == 1 and logits.shape == weights.shape
+        T, E = logits.shape
+        self._run(f"route_topk {T}x{E}", T * E * 8, 8 * T * E, None, self.lib.llmrs_route_topk, self._stream(), _p(logits),
+                  logits.stride(0), _p(weights), weights.stride(0), T, E, int(top), int(bool(renormalize)))
+
+    def act_weight(self, out: torch.Tensor, up: torch.Tensor, weights: Optional[torch.Tensor], ff: int) -> None:
+        """out[t, c] = relu(up[t, c])^2 * (weights[t, c // ff] if weights is given); up, weights float32."""
+        T, N = up.shape
+        assert up.dtype == torch.float32 and up.stride(1) == 1 and out.shape == up.shape and out.stride(1) == 1 and N % ff == 0
+        assert weights is None or (weights.dtype == torch.float32 and weights.stride(1) == 1 and tuple(weights.shape) == (T, N // ff))
+        self._run(f"act_weight {T}x{N}", T * N * (4 + out.element_size()), 3 * T * N, None,
+                  self.lib.llmrs_act_weight, self._stream(), _code(out.dtype), _p(up), up.stride(0), _p(weights),
+                  0 if weights is None else weights.stride(0), int(ff), T, N, 0, _p(out), out.stride(0))
 
     def scan_carry_floats(self, n_tokens: int, n_entries: int, longest: int, per_place: int) -> int:
         """Room (in floats) for what the chunks of a recurrence hand on, `per_place` floats for each chunk's place;

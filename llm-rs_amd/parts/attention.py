@@ -14,8 +14,11 @@ the product.  No biases.
 Options for mixers that prepare q and k otherwise (all off for Llama): `value_dim` (values of another width than
 keys), `bias` (q, k and v have biases), `qk_norm_eps` (q and k are divided by their root mean square over the head,
 with this eps, no weight), `distance` = "log" (a per-head penalty r1 ln(1 + r2 (i - j)) taken off the scaled score,
-with the head's numbers in two tensors), `names` (the leaves of the tensors' names).  With any of them the q/k/v
-product leaves 32-bit sums, and one kernel adds the biases, norms q and k and writes k and v into their pages.
+with the head's numbers in two tensors), `softcap` (the scaled score s becomes softcap tanh(s / softcap)),
+`keep_first` (with a window, the request's first so many keys stay visible at their true positions; their pages stay in
+the cache), `o_bias` (the output projection has a bias), `names` (the leaves of the tensors' names).  With any of them
+the q/k/v product leaves 32-bit sums, and one kernel adds the biases, norms q and k, rotates them (a rotation that the
+kernels fuse, angles in 32-bit) and writes k and v into their pages.
 
 The rotation kernels pair neighbours (2i, 2i+1).  Where the encoding pairs
 (i, i + rotary_dim/2), the rows of Wq and Wk are reordered within each head at
@@ -64,17 +67,24 @@ class Attention(Mixer):
         self.distance = p.get("distance")
         if self.distance not in (None, "log"):
             raise ValueError(f"unknown distance penalty {self.distance!r} (known: log)")
+        self.softcap = float(p.get("softcap") or 0.0)
+        self.keep_first = int(p.get("keep_first") or 0) if self.window > 0 else 0
+        self.has_o_bias = bool(p.get("o_bias", False))
+        if self.softcap < 0 or self.keep_first < 0:
+            raise ValueError("softcap and keep_first must not be negative")
         # q and k are prepared by a kernel of their own between the product and attention
-        self.prepared = self.has_bias or self.qk_norm_eps > 0 or self.distance is not None or self.value_dim != self.head_dim
-        if self.prepared and self.position is not None:
-            raise ValueError("a position encoding together with biases, a q/k norm, a distance penalty or values of another width is not built")
+        self.prepared = (self.has_bias or self.qk_norm_eps > 0 or self.distance is not None or self.value_dim != self.head_dim
+                         or self.softcap > 0 or self.keep_first > 0)
+        if self.prepared and self.position is not None and self.position.rotary() is None:
+            raise ValueError("a position encoding that is no rotation together with biases, a q/k norm, a distance penalty, a soft cap, "
+                             "kept first keys or values of another width is not built")
         leaves = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
-                  "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "r1": "r1", "r2": "r2",
+                  "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias", "r1": "r1", "r2": "r2",
                   **(p.get("names") or {})}
         self.names = {key: self.name(leaf) for key, leaf in leaves.items()}
         self.w_qkv = None
         self.w_o = None
-        self.bias = self.r1 = self.r2 = None
+        self.bias = self.o_bias = self.r1 = self.r2 = None
 
     def tensors(self):
         n = self.names
@@ -87,6 +97,8 @@ class Attention(Mixer):
             if self.kv_proj:
                 t[n["k_bias"]] = TensorSpec((self.kv_size,))
                 t[n["v_bias"]] = TensorSpec((self.v_size,))
+        if self.has_o_bias:
+            t[n["o_bias"]] = TensorSpec((self.hidden,))
         if self.distance is not None:
             t[n["r1"]] = TensorSpec((self.heads,), "normal:0.5:0.2")
             t[n["r2"]] = TensorSpec((self.heads,), "normal:0.5:0.05")     # 1 + r2 (i - j) must stay positive
@@ -112,8 +124,12 @@ class Attention(Mixer):
             parts += [self._pair_neighbours(get("k"), self.kv_heads), get("v")]
         self.w_qkv = torch.cat(parts, dim=0).contiguous()
         self.w_o = get("o")
-        if self.has_bias:       # added to the 32-bit sums: kept in 32-bit, side by side as the product's columns are
-            self.bias = torch.cat([get32("q_bias")] + ([get32("k_bias"), get32("v_bias")] if self.kv_proj else [])).contiguous()
+        if self.has_bias:       # added to the 32-bit sums: kept in 32-bit, side by side as the product's columns are (and reordered as its rows are)
+            pair = lambda b, heads: self._pair_neighbours(b.unsqueeze(1), heads).squeeze(1)
+            self.bias = torch.cat([pair(get32("q_bias"), self.heads)] +
+                                  ([pair(get32("k_bias"), self.kv_heads), get32("v_bias")] if self.kv_proj else [])).contiguous()
+        if self.has_o_bias:
+            self.o_bias = get32("o_bias")
         if self.distance is not None:
             self.r1, self.r2 = get32("r1"), get32("r2")
         if self.position is not None:
@@ -129,19 +145,23 @@ class Attention(Mixer):
             out[n["v"]] = v.contiguous()
         if self.has_bias:
             b = self.bias.cpu()
-            out[n["q_bias"]] = b[:self.q_size].contiguous()
+            unpair = lambda x, heads: self._pair_neighbours(x.unsqueeze(1), heads, undo=True).squeeze(1).contiguous()
+            out[n["q_bias"]] = unpair(b[:self.q_size], self.heads)
             if self.kv_proj:
-                out[n["k_bias"]] = b[self.q_size:self.q_size + self.kv_size].contiguous()
+                out[n["k_bias"]] = unpair(b[self.q_size:self.q_size + self.kv_size], self.kv_heads)
                 out[n["v_bias"]] = b[self.q_size + self.kv_size:].contiguous()
+        if self.has_o_bias:
+            out[n["o_bias"]] = self.o_bias.cpu()
         if self.distance is not None:
             out[n["r1"]], out[n["r2"]] = self.r1.cpu(), self.r2.cpu()
         return out
 
     def cache_need(self):
-        return PagedKV(self.kv_heads, self.head_dim, self.window, self.value_dim if self.value_dim != self.head_dim else 0)
+        return PagedKV(self.kv_heads, self.head_dim, self.window, self.value_dim if self.value_dim != self.head_dim else 0, self.keep_first)
 
     def _forward_prepared(self, ctx, x, h, cache):
-        """The product's 32-bit sums -> biases, unit norm of q and k, cache write -> attention with the distance penalty."""
+        """The product's 32-bit sums -> biases, unit norm and rotation of q and k, cache write -> attention with the
+        distance penalty, the soft cap and the kept first keys."""
         k = kernels()
         T = x.shape[0]
         write = self.kv_proj and cache.writes
@@ -150,8 +170,10 @@ class Attention(Mixer):
         sums = ctx.workspace("attn.sums", (T, self.w_qkv.shape[0]), torch.float32)
         k.gemm(x, self.w_qkv, sums, EPI_STORE_F32, ctx.gemm_workspace(x, self.w_qkv))
         q = ctx.workspace("attn.qkv", (T, self.q_size), self.dtype)
+        rotary = self.position.rotary() if self.position is not None else None
+        inv_freq, rotary_dim = (None, 0) if rotary is None else rotary[:2]
         k.qkv_finish(sums, self.bias, q, ctx.slot_maps[g], cache.k, cache.v, self.heads, n_kv, self.head_dim, self.value_dim,
-                     cache.page_size, cache.num_pages, write, self.qk_norm_eps)
+                     cache.page_size, cache.num_pages, write, self.qk_norm_eps, ctx.positions, inv_freq, rotary_dim)
         o = ctx.workspace("attn.out", (T, self.o_size), self.dtype)
         need = k.attention_scratch_floats(ctx.n_entries, self.heads, max(self.head_dim, self.value_dim), ctx.max_seq_len,
                                           self.kv_heads, ctx.n_single) if ctx.n_single else 0
@@ -159,8 +181,10 @@ class Attention(Mixer):
         k.attention(q, o, cache.k, cache.v, ctx.block_tables[g], ctx.token_entry, ctx.positions, ctx.q_starts, ctx.seq_lens,
                     self.heads, self.kv_heads, self.head_dim, cache.page_size, cache.num_pages, self.window, self.scale,
                     scratch, ctx.max_seq_len, ctx.n_single, self._keys_for_the_split(ctx), value_dim=self.value_dim,
-                    distance=None if self.distance is None else (self.r1, self.r2))
+                    distance=None if self.distance is None else (self.r1, self.r2), softcap=self.softcap, keep_first=self.keep_first)
         k.gemm(o, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(o, self.w_o))
+        if self.has_o_bias:
+            k.add_bias_rows(h, self.o_bias)
         ctx.note_left(h, None)
 
     def takes_normed_rows(self, ctx, rows):
@@ -232,8 +256,10 @@ class Attention(Mixer):
                     ctx.q_starts, ctx.seq_lens, self.heads, self.kv_heads, self.head_dim, cache.page_size,
                     cache.num_pages, self.window, self.scale, scratch, ctx.max_seq_len, ctx.n_single,
                     self._keys_for_the_split(ctx))
-        leave = ctx.room_for_next_norm(h, self.w_o)
+        leave = ctx.room_for_next_norm(h, self.w_o) if not self.has_o_bias else None
         k.gemm(o, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(o, self.w_o), **({} if leave is None else {"leave": leave}))
+        if self.has_o_bias:
+            k.add_bias_rows(h, self.o_bias)
         ctx.note_left(h, leave)
 
 

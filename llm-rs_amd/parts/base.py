@@ -99,6 +99,16 @@ class Norm(Part):
         """out[i] = norm(h[rows[i]]) (rows None: every row)."""
         raise NotImplementedError
 
+    def forward_clearing(self, ctx, h: torch.Tensor, out: torch.Tensor, zero: torch.Tensor) -> None:
+        """`forward` over every row, and `zero` ([T, size] float32, where a sublayer will add its result) cleared: a
+        norm whose kernel can do both in one launch does."""
+        self.forward(ctx, h, out)
+        zero.zero_()
+
+    def add_normed(self, ctx, y: torch.Tensor, h: torch.Tensor) -> None:
+        """h += norm(y), both float32 [T, size]: the norm of a sublayer's output on its way into the stream."""
+        raise NotImplementedError(f"{type(self).__name__} cannot norm a sublayer's output into the stream")
+
     def deferred_weight(self) -> Optional[torch.Tensor]:
         """For a norm of the form x / rms(x) * weight: the float32 weight, which lets the product before it
         prepare its rows and the product after it finish them (`kernels.NextNorm`, `kernels.NormedRows`);

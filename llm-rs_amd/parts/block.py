@@ -2,8 +2,10 @@
 (src/arch/llama.rs:152-170).  Another arrangement (one norm for two parallel
 halves, norms after the parts) is another subclass of `Block`, registered under
 its own name; the parts it needs beyond these four come under the names the
-layer's spec gives them in `extra`."""
+layer's spec gives them in `extra`.  "sandwich": a norm before and after each half."""
 from __future__ import annotations
+
+import torch
 
 from .base import Block, register_block
 
@@ -32,3 +34,37 @@ class PreNormBlock(Block):
 
 
 register_block("prenorm", PreNormBlock)
+
+
+class SandwichBlock(Block):
+    """A norm before and after each sublayer: h += post_mixer_norm(mixer(mixer_norm(h))), then, where the layer has a
+    feed-forward, h += post_feed_forward_norm(feed_forward(feed_forward_norm(h))).  The sublayer adds its result into
+    a cleared 32-bit buffer of the stream's shape; the norm after it reads that and adds into the stream, in 32-bit."""
+    needs = ("mixer", "mixer_norm", "post_mixer_norm")
+
+    def __init__(self, named):
+        super().__init__(named)
+        self.post_mixer_norm = self.named["post_mixer_norm"]
+        self.post_feed_forward_norm = self.named.get("post_feed_forward_norm")
+        if self.feed_forward is not None and (self.feed_forward_norm is None or self.post_feed_forward_norm is None):
+            raise ValueError("a feed-forward between two norms needs both of them")
+
+    def _half(self, ctx, h, norm, post, run) -> None:
+        T, D = h.shape
+        x = ctx.workspace("block.x", (T, D), self.mixer.dtype)
+        y = ctx.workspace("block.y", (T, D), torch.float32)
+        ctx.note_left(h, None)
+        ctx.upcoming_norm = None
+        norm.forward_clearing(ctx, h, x, y)
+        run(x, y)
+        post.add_normed(ctx, y, h)
+
+    def forward(self, ctx, h, cache):
+        self._half(ctx, h, self.mixer_norm, self.post_mixer_norm, lambda x, y: self.mixer.forward(ctx, x, y, cache))
+        if self.feed_forward is not None:
+            self._half(ctx, h, self.feed_forward_norm, self.post_feed_forward_norm, lambda x, y: self.feed_forward.forward(ctx, x, y))
+        ctx.note_left(h, None)
+        ctx.upcoming_norm = None
+
+
+register_block("sandwich", SandwichBlock)

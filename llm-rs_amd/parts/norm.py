@@ -10,27 +10,36 @@ from .base import Norm, TensorSpec, place, register_norm
 
 
 class RMSNorm(Norm):
+    """`tensor`: the leaf of the weight's name ("weight"); "" when the prefix itself is the name."""
     graph_safe = True
 
     def __init__(self, spec, dtype):
         super().__init__(spec, dtype)
         self.size = int(spec.params["size"])
         self.eps = float(spec.params["eps"])
+        leaf = spec.params.get("tensor", "weight")
+        self.weight_name = self.name(leaf) if leaf else self.prefix
         self.weight = None
 
     def tensors(self):
-        return {self.name("weight"): TensorSpec((self.size,), "norm")}
+        return {self.weight_name: TensorSpec((self.size,), "norm")}
 
     def load(self, tensors, device):
         # The reference wants norm weights in 32-bit (ops.metal:972); whatever the
         # file stores, the kernel multiplies by a float32 weight.
-        self.weight = place(tensors[self.name("weight")], device, torch.float32)
+        self.weight = place(tensors[self.weight_name], device, torch.float32)
 
     def export(self):
-        return {self.name("weight"): self.weight.cpu()}
+        return {self.weight_name: self.weight.cpu()}
 
     def forward(self, ctx, h, out, rows=None):
         kernels().rmsnorm(out, h, self.weight, self.eps, rows)
+
+    def forward_clearing(self, ctx, h, out, zero):
+        kernels().group_rmsnorm(out, h, self.weight, self.eps, 1, zero=zero)       # (one group: this norm; clears on the way)
+
+    def add_normed(self, ctx, y, h):
+        kernels().rmsnorm_sum(h, [(y, None, self.weight)], 1.0, self.eps)
 
     def deferred_weight(self):
         return self.weight

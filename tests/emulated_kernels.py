@@ -109,25 +109,136 @@ class EmulatedKernels(Kernels):
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
                   n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1,
-                  single_keys=0):
+                  single_keys=0, value_dim=0, distance=None, softcap=0.0, keep_first=0):
         T = q.shape[0]
+        v_dim = value_dim or head_dim
         kc = k_cache.view(num_pages, n_kv_heads, page_size, head_dim).float()
-        vc = v_cache.view(num_pages, n_kv_heads, head_dim, page_size).float()
+        vc = v_cache.view(num_pages, n_kv_heads, v_dim, page_size).float()
         rep = n_heads // n_kv_heads
         for t in range(T):
             pos = int(positions[t])
             table = block_table[int(token_entry[t])]
             lo = max(0, pos + 1 - window) if window > 0 else 0
-            js = torch.arange(lo, pos + 1)
+            js = torch.cat([torch.arange(0, min(keep_first, lo)), torch.arange(lo, pos + 1)])
             pages, offs = table[js // page_size].long(), js % page_size
+            assert int(pages.min()) >= 0, "a visible key's page was given back"
             keys = kc[pages, :, offs, :]                       # [n, kv, d]
             vals = vc[pages, :, :, offs]                       # [n, kv, d]
             qt = q[t, :n_heads * head_dim].view(n_heads, head_dim).float()
             for h in range(n_heads):
                 g = h // rep
                 s = (keys[:, g, :] @ qt[h]) * scale
+                if softcap > 0:
+                    s = softcap * torch.tanh(s / softcap)
+                if distance is not None:
+                    s = s - distance[0][h] * torch.log1p(distance[1][h] * (pos - js).float())
                 p = torch.softmax(s, dim=0)
-                out[t, h * head_dim:(h + 1) * head_dim] = (p @ vals[:, g, :]).to(out.dtype)
+                out[t, h * v_dim:(h + 1) * v_dim] = (p @ vals[:, g, :]).to(out.dtype)
+
+    def group_rmsnorm(self, out, x, weight, eps, groups, rows=None, w_in=None, zero=None, combined=None, mix=None):
+        assert x.dim() == 2 and w_in is None and combined is None and mix is None, "one stream only"
+        src = x if rows is None else x[rows.long()]
+        parts = src.view(src.shape[0], groups, -1)
+        inv = 1.0 / torch.sqrt((parts * parts).mean(-1, keepdim=True) + eps)
+        out.copy_(((parts * inv).view(src.shape) * weight).to(out.dtype))
+        if zero is not None:
+            zero.zero_()
+
+    def qkv_finish(self, sums, bias, q, slot_map, k_cache, v_cache, n_heads, n_kv_heads, head_dim, v_dim, page_size, num_pages,
+                   write_kv, eps, positions=None, inv_freq=None, rotary_dim=0):
+        T = sums.shape[0]
+        x = sums + bias if bias is not None else sums.clone()
+        nq, nk = n_heads * head_dim, n_kv_heads * head_dim
+        qk = x[:, :nq + nk].reshape(T, n_heads + n_kv_heads, head_dim)
+        if eps > 0:
+            qk = qk / torch.sqrt((qk * qk).mean(-1, keepdim=True) + eps)
+        if rotary_dim:
+            angle = positions.float()[:, None] * inv_freq[None, :]
+            cos, sin = torch.cos(angle)[:, None, :], torch.sin(angle)[:, None, :]
+            a, b = qk[..., 0:rotary_dim:2].clone(), qk[..., 1:rotary_dim:2].clone()
+            qk[..., 0:rotary_dim:2], qk[..., 1:rotary_dim:2] = a * cos - b * sin, b * cos + a * sin
+        q.copy_(qk[:, :n_heads].reshape(T, nq).to(q.dtype))
+        if not write_kv:
+            return
+        kc = k_cache.view(num_pages, n_kv_heads, page_size, head_dim)
+        vc = v_cache.view(num_pages, n_kv_heads, v_dim, page_size)
+        page, off = (slot_map // page_size).long(), (slot_map % page_size).long()
+        vals = x[:, nq + nk:].reshape(T, n_kv_heads, v_dim)
+        for t in range(T):
+            kc[page[t], :, off[t], :] = qk[t, n_heads:].to(kc.dtype)
+            vc[page[t], :, :, off[t]] = vals[t].to(vc.dtype)
+
+    def add_bias_rows(self, rows, bias):
+        rows.add_(bias)
+
+    def causal_conv_silu(self, sums, taps, bias, state, q_starts, slots, token_entry, channels, out):
+        K = taps.shape[1]
+        for e in range(slots.numel()):
+            t0, t1 = int(q_starts[e]), int(q_starts[e + 1])
+            st = state[int(slots[e])][:(K - 1) * channels].view(K - 1, channels)
+            xs = torch.cat([st, sums[t0:t1, :channels]], dim=0)          # the last K - 1 inputs, then this portion's
+            for i in range(t1 - t0):
+                acc = (taps.T * xs[i:i + K]).sum(0) + (bias if bias is not None else 0.0)
+                out[t0 + i] = (acc / (1.0 + torch.exp(-acc))).to(out.dtype)
+            if K > 1:
+                st.copy_(xs[xs.shape[0] - (K - 1):].clone())
+
+    def silu_columns(self, x, col0, n):
+        v = x[:, col0:col0 + n]
+        v.copy_(v / (1.0 + torch.exp(-v)))
+
+    def delta_prepare(self, q, k, a, b, A_log, dt_bias, heads, qk_heads, dk, unit_eps):
+        T = q.shape[0]
+        for x, scale in ((q, dk ** -0.5), (k, 1.0)):
+            v = x.reshape(T, qk_heads, dk)
+            x.copy_((v / torch.sqrt((v * v).sum(-1, keepdim=True) + unit_eps) * scale).reshape(T, -1))
+        z = a.reshape(T, heads, dk) + dt_bias.view(heads, dk)
+        soft = torch.where(z > 20.0, z, torch.log1p(torch.exp(torch.clamp(z, max=20.0))))
+        a.copy_(torch.exp(-torch.exp(A_log)[None, :, None] * soft).reshape(T, -1))
+        b.copy_(1.0 / (1.0 + torch.exp(-b)))
+
+    def linear_scan(self, q, k, v, state, q_starts, slots, heads, qk_heads, dk, dv, out, decay=None, g=None, beta=None):
+        rep = heads // qk_heads
+        for e in range(slots.numel()):
+            S = state[int(slots[e])][:heads * dk * dv].view(heads, dk, dv)
+            for t in range(int(q_starts[e]), int(q_starts[e + 1])):
+                qt = q[t].view(qk_heads, dk).repeat_interleave(rep, dim=0)
+                kt = k[t].view(qk_heads, dk).repeat_interleave(rep, dim=0)
+                vt = v[t].view(heads, dv)
+                if g is not None:
+                    S.mul_(g[t].view(heads, dk)[:, :, None])
+                elif decay is not None:
+                    S.mul_(decay[:, None, None])
+                u = vt if beta is None else beta[t][:, None] * (vt - torch.einsum("hkv,hk->hv", S, kt))
+                S.add_(kt[:, :, None] * u[:, None, :])
+                out[t] = torch.einsum("hkv,hk->hv", S, qt).reshape(-1)
+
+    def gated_rmsnorm(self, out, x, gate, weight, group, eps):
+        T, W = x.shape
+        parts = x.reshape(T, W // group, group)
+        y = (parts / torch.sqrt((parts * parts).mean(-1, keepdim=True) + eps)).reshape(T, W)
+        w = weight if weight.numel() == W else weight.repeat(W // group)
+        out.copy_((y * w / (1.0 + torch.exp(-gate))).to(out.dtype))
+
+    def rmsnorm_sum(self, out, inputs, coef, eps):
+        for x, bias, weight in inputs:
+            v = x if bias is None else x + bias
+            out.add_(coef * v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * weight)
+
+    def route_topk(self, logits, weights, top, renormalize=False):
+        scores = torch.softmax(logits, dim=-1)
+        weights.zero_()
+        for t in range(logits.shape[0]):
+            chosen = sorted(range(logits.shape[1]), key=lambda e: (-float(scores[t, e]), e))[:top]
+            total = sum(float(scores[t, e]) for e in chosen) if renormalize else 1.0
+            for e in chosen:
+                weights[t, e] = scores[t, e] / total
+
+    def act_weight(self, out, up, weights, ff):
+        y = torch.clamp(up, min=0.0) ** 2
+        if weights is not None:
+            y = y * weights.repeat_interleave(ff, dim=1)
+        out.copy_(y.to(out.dtype))
 
     def argmax_rows(self, logits, out, scratch=None):
         for i in range(logits.shape[0]):
