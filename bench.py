@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b|prompts|long|widths|portions|tuvodra]
+    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b|prompts|long|widths|portions|tuvodra|lilatar]
 
 The default run (`decode8b`) is the Llama-3.1-8B shape with random bfloat16 weights: 8
 requests, each with 2,048 tokens of context in the cache, decode K steps through the
@@ -33,6 +33,10 @@ The other workloads print one line of the same form each:
             share seen at the same number of rows.
   portions  the attention of one request's prompt portion of 2,048 tokens alone (8B shape's heads), over caches of
             2,048 (the whole prompt: causal) to 131,072 keys: TFLOP/s for each; value = the one over 65,536 keys.
+  tuvodra   the Tuvodra decoder at the 1B and 8B widths beside a Llama decoder of equal widths and depth: a prompt of
+            2,048 tokens and a decode step of 8 requests over 2,048 tokens for each.
+  lilatar   the same for the Lilatar decoder (linear attention, windowed attention beside a gated delta rule,
+            dense and routed squared-relu feed-forwards).
 With LLM_PERF set in the environment every kernel call is timed by itself and a table
 by kernel goes to stderr (the reference's switch, src/backend/metal/mod.rs:235,321-400).
 """
@@ -63,7 +67,7 @@ LLAMA_8B = _llama(32, 4096, 32, 8, 128, 14336, 8.0, False)
 LLAMA_1B = _llama(16, 2048, 32, 8, 64, 8192, 32.0, True)
 LLAMA_70B = _llama(80, 8192, 64, 8, 128, 28672, 8.0, False)
 SHAPES = {"Llama-3.1-8B shape": LLAMA_8B, "Llama-3.2-1B shape": LLAMA_1B, "Llama-3.1-70B shape": LLAMA_70B}
-WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts", "long", "widths", "portions", "tuvodra")
+WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts", "long", "widths", "portions", "tuvodra", "lilatar")
 
 
 def flat_config(model: str, layers_run: int, global_batch: int, seq_len: int, page_size: int, **more) -> dict:
@@ -550,20 +554,15 @@ def tuvodra_shape(width, heads, kv_heads, dim, ff, window, repeats, vocab=128256
             "norm": {"eps": 1e-6, "groups": 4}, "layers": [dict(l) for _ in range(repeats) for l in three]}
 
 
-def run_tuvodra(args) -> dict:
-    """Prompt and decode throughput of the Tuvodra decoder at two widths, each beside a Llama decoder of the same
-    width, heads, feed-forward and number of layers (random weights both)."""
+def run_beside_llama(args, pairs: dict, layers_run: int) -> dict:
+    """Prompt and decode throughput of each model of `pairs` ({size: {name: configuration}}, random weights)."""
     from llm_rs_amd import StepEntry
     from llm_rs_amd.kernels import kernels
-    repeats = max(1, (args.layers or 6) // 3)
     T, batch, context = args.prefill_tokens, args.batch, args.context
-    sizes = {"1B widths": (LLAMA_1B, 2048, 32, 8, 64, 8192), "8B widths": (LLAMA_8B, 4096, 32, 8, 128, 14336)}
     points = {}
-    for size, (llama, width, heads, kv_heads, dim, ff) in sizes.items():
+    for size, pair in pairs.items():
         if args.only_size and args.only_size not in size:
             continue
-        pair = {"tuvodra": tuvodra_shape(width, heads, kv_heads, dim, ff, args.window, repeats),
-                "llama": dict(llama, num_hidden_layers=3 * repeats)}
         for name, shape in pair.items():
             b = Bench(args, shape, batch * (context + 256) // 16 + T // 16 + 64, max(batch, 8), max(T, 2048))
             engine = b.engine
@@ -595,11 +594,59 @@ def run_tuvodra(args) -> dict:
             gc.collect()
             import torch
             torch.cuda.empty_cache()
+    return points
+
+
+def run_tuvodra(args) -> dict:
+    """Prompt and decode throughput of the Tuvodra decoder at two widths, each beside a Llama decoder of the same
+    width, heads, feed-forward and number of layers (random weights both)."""
+    repeats = max(1, (args.layers or 6) // 3)
+    sizes = {"1B widths": (LLAMA_1B, 2048, 32, 8, 64, 8192), "8B widths": (LLAMA_8B, 4096, 32, 8, 128, 14336)}
+    pairs = {size: {"tuvodra": tuvodra_shape(width, heads, kv_heads, dim, ff, args.window, repeats), "llama": dict(llama, num_hidden_layers=3 * repeats)}
+             for size, (llama, width, heads, kv_heads, dim, ff) in sizes.items()}
+    points = run_beside_llama(args, pairs, 3 * repeats)
     first = next(iter(points.values()))
     line = base_line("decode_tokens_per_s", first["decode_tokens_per_s"], args.steps, args.warmup, first["decode_ms_per_step"] * 1e-3, args.dtype,
                      {"model": "Tuvodra (minGRU, selective scan, windowed attention + feed-forward, in threes) beside Llama of equal widths",
-                      "global_batch": batch, "seq_len": context, "parallelism": "single GPU", "layers_run": 3 * repeats,
-                      "prefill_tokens": T, "window": args.window, "streams": 4, "norm_groups": 4, "page_size": 16})
+                      "global_batch": args.batch, "seq_len": args.context, "parallelism": "single GPU", "layers_run": 3 * repeats,
+                      "prefill_tokens": args.prefill_tokens, "window": args.window, "streams": 4, "norm_groups": 4, "page_size": 16})
+    line["points"] = points
+    return line
+
+
+def lilatar_shape(width, heads, kv_heads, dim, ff, window, repeats, experts, top, vocab=128256):
+    """Layers in threes: linear attention with a dense feed-forward, then two layers of windowed attention beside a
+    gated delta rule with a mixture of experts whose chosen experts together are as wide as the dense feed-forward;
+    heads and widths of the Llama shape of that width."""
+    wide = max(dim, 128)                # heads of the two recurrent mixers
+    lin = {"heads": width // wide, "dim": wide, "vdim": wide, "decay": [1.0 - 2.0 ** -(3 + 5 * i / max(width // wide - 1, 1)) for i in range(width // wide)]}
+    par = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "softcap": 30.0,
+                    "mask": {"size": window, "keep_first": 4},
+                    "rot": {"dims": dim // 2, "base": 10000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}},
+           "right": {"heads": width // wide, "kv_heads": width // wide, "dim": wide, "vdim": wide, "conv": 4, "decay_rank": width // 16, "gate_rank": width // 16}}
+    routed = {"kind": "moe", "expert": {"ff": ff // top}, "router": {"experts": experts, "top": top}}
+    three = [{"type": "lightning", "mixer": lin, "mlp": {"kind": "dense", "ff": ff}},
+             {"type": "parallel", "mixer": par, "mlp": routed}, {"type": "parallel", "mixer": par, "mlp": routed}]
+    import copy
+    return {"architecture": "Lilatar", "vocab": vocab, "width": width, "logit_scale": 1.0, "norm": {"eps": 1e-6},
+            "layers": [copy.deepcopy(l) for _ in range(repeats) for l in three]}
+
+
+def run_lilatar(args) -> dict:
+    """Prompt and decode throughput of the Lilatar decoder at two widths, each beside a Llama decoder of the same
+    width, heads, feed-forward and number of layers (random weights both)."""
+    repeats = max(1, (args.layers or 6) // 3)
+    sizes = {"1B widths": (LLAMA_1B, 2048, 32, 8, 64, 8192), "8B widths": (LLAMA_8B, 4096, 32, 8, 128, 14336)}
+    pairs = {size: {"lilatar": lilatar_shape(width, heads, kv_heads, dim, ff, args.window, repeats, args.experts, args.top),
+                    "llama": dict(llama, num_hidden_layers=3 * repeats)}
+             for size, (llama, width, heads, kv_heads, dim, ff) in sizes.items()}
+    points = run_beside_llama(args, pairs, 3 * repeats)
+    first = next(iter(points.values()))
+    line = base_line("decode_tokens_per_s", first["decode_tokens_per_s"], args.steps, args.warmup, first["decode_ms_per_step"] * 1e-3, args.dtype,
+                     {"model": "Lilatar (linear attention + dense feed-forward, then twice windowed attention beside a gated delta rule + experts) "
+                               "beside Llama of equal widths",
+                      "global_batch": args.batch, "seq_len": args.context, "parallelism": "single GPU", "layers_run": 3 * repeats,
+                      "prefill_tokens": args.prefill_tokens, "window": args.window, "experts": args.experts, "top": args.top, "page_size": 16})
     line["points"] = points
     return line
 
@@ -621,8 +668,10 @@ def main() -> int:
     ap.add_argument("--requests", type=int, default=256, help="serve1b: requests submitted at once")
     ap.add_argument("--new-tokens", type=int, default=256, help="serve1b: tokens generated for each request")
     ap.add_argument("--max-batch-tokens", type=int, default=2048, help="serve1b: tokens a scheduler step may run")
-    ap.add_argument("--window", type=int, default=1024, help="tuvodra: keys an attention layer sees")
-    ap.add_argument("--only-size", default="", help="tuvodra: run one of the sizes only (1B or 8B)")
+    ap.add_argument("--window", type=int, default=1024, help="tuvodra, lilatar: keys an attention layer sees")
+    ap.add_argument("--only-size", default="", help="tuvodra, lilatar: run one of the sizes only (1B or 8B)")
+    ap.add_argument("--experts", type=int, default=16, help="lilatar: experts of a routed feed-forward")
+    ap.add_argument("--top", type=int, default=4, help="lilatar: experts a token uses")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -631,7 +680,7 @@ def main() -> int:
     args.steps = args.steps if args.steps is not None else (8 if heavy else 64)
     args.warmup = args.warmup if args.warmup is not None else (2 if heavy else 8)
     line = {"decode8b": run_decode8b, "serve1b": run_serve1b, "mixed70b": run_mixed70b, "sizes": run_sizes, "sizes1b": run_sizes,
-            "prompts": run_prompts, "long": run_long, "widths": run_widths, "portions": run_portions, "tuvodra": run_tuvodra}[args.workload](args)
+            "prompts": run_prompts, "long": run_long, "widths": run_widths, "portions": run_portions, "tuvodra": run_tuvodra, "lilatar": run_lilatar}[args.workload](args)
     from llm_rs_amd.kernels import kernels
     if kernels().times is not None:         # LLM_PERF: what was still to be shown of the per-kernel table
         kernels().times.dump()

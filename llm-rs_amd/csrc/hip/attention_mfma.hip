@@ -74,9 +74,26 @@ __device__ __forceinline__ float other_half(float x) {
 #define ATTN_WIDE_FROM_KEYS 32768        // tiles of eight waves from this bound on the step's lengths
 // With `far` (the same in all lanes) a penalty that grows with the logarithm of the distance is taken off first:
 // S c - r1 log2(1 + r2 (pos - key)), which is (score - r1 ln(1 + r2 d)) log2(e); r1 and r2 are the column's head's.
+// With `cap` > 0 (the same in all lanes) the scaled score s is first bent into (-cap, cap): cap tanh(s / cap), with
+// tanh(x) = 1 - 2 / (1 + 2^(2 x log2 e)) on the hardware's exponential and reciprocal; `cap_in` is scale / cap.
+// `keep`: keys below it stay visible though they lie before lo.
+struct ScoreBend {
+    float cap, cap_in;      // 0, 0: scores as they are
+    int keep;
+};
+__device__ __forceinline__ float bent_score_log2(float dot, const ScoreBend& b) {
+    float e = __builtin_amdgcn_exp2f(dot * b.cap_in * (2.0f * 1.44269504088896341f));
+    float th = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e);
+    return b.cap * 1.44269504088896341f * th;
+}
 __device__ __forceinline__ bool softmax_tile(f32x16& S, float& m, float& l, int t0, int pos, int lo,
                                              int h, float c, float& alpha, bool edge,
-                                             bool far = false, float r1 = 0.0f, float r2 = 0.0f) {
+                                             bool far = false, float r1 = 0.0f, float r2 = 0.0f, ScoreBend bend = ScoreBend{0.0f, 0.0f, 0}) {
+    if (bend.cap > 0.0f) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) S[i] = bent_score_log2(S[i], bend);
+        c = 1.0f;
+    }
     if (far) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
@@ -90,7 +107,7 @@ __device__ __forceinline__ bool softmax_tile(f32x16& S, float& m, float& l, int 
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             int key = t0 + 16 * (i >> 3) + 8 * h + 4 * ((i >> 2) & 1) + (i & 3);
-            S[i] = (key > pos || key < lo) ? -INFINITY : S[i];
+            S[i] = (key > pos || (key < lo && key >= bend.keep)) ? -INFINITY : S[i];
         }
     }
     float mx = S[0];
@@ -127,7 +144,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
                                              const int* __restrict__ table, int table_width, int num_pages,
                                              int n_kv, int kvh, int t_begin, int t_end, int pos, int lo, float scale,
                                              bool have_pages = false, int first_pages = 0,
-                                             bool far = false, float r1 = 0.0f, float r2 = 0.0f) {
+                                             bool far = false, float r1 = 0.0f, float r2 = 0.0f, ScoreBend bend = ScoreBend{0.0f, 0.0f, 0}) {
     int lane = threadIdx.x & 63;
     int r = lane & 31, h = lane >> 5;
     float scale_log2e = scale * 1.44269504088896341f;
@@ -197,7 +214,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
             vf[dt][0] = *(const bf16x8*)(vp0 + dt * 32 * 16);
             vf[dt][1] = *(const bf16x8*)(vp1 + dt * 32 * 16);
         }
-        bool moved = softmax_tile(S, m, l, t0, pos, lo, h, scale_log2e, alpha_out, __any(t0 + 31 > pos || t0 < lo), far, r1, r2);
+        bool moved = softmax_tile(S, m, l, t0, pos, lo, h, scale_log2e, alpha_out, __any(t0 + 31 > pos || t0 < lo), far, r1, r2, bend);
         float alpha = alpha_out;
         bf16x8 pf[2];
 #pragma unroll
@@ -260,9 +277,15 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(const bf16* __restrict_
 #pragma unroll
         for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
     float m = -INFINITY, l = 0.0f;
+    const ScoreBend bend{a.softcap, a.softcap > 0.0f ? a.scale / a.softcap : 0.0f, a.keep_first};
+    // the first keys that stay visible, where they lie before the window's tiles (those among them pass the mask there)
+    if (a.keep_first > 0 && t_begin > 0)
+        attend_range<HD>(qf, O, m, l, kc, vc, block_table + (size_t)e * a.table_width, a.table_width, a.num_pages,
+                         a.n_kv_heads, kvh, 0, min(a.keep_first, t_begin), pos, lo, a.scale, false, 0,
+                         a.dist_r1 != nullptr, a.dist_r1 ? a.dist_r1[head] : 0.0f, a.dist_r1 ? a.dist_r2[head] : 0.0f, bend);
     attend_range<HD>(qf, O, m, l, kc, vc, block_table + (size_t)e * a.table_width, a.table_width, a.num_pages,
                      a.n_kv_heads, kvh, t_begin, t_end, pos, lo, a.scale, false, 0,
-                     a.dist_r1 != nullptr, a.dist_r1 ? a.dist_r1[head] : 0.0f, a.dist_r1 ? a.dist_r2[head] : 0.0f);
+                     a.dist_r1 != nullptr, a.dist_r1 ? a.dist_r1[head] : 0.0f, a.dist_r1 ? a.dist_r2[head] : 0.0f, bend);
     if (!cvalid) return;
     float inv = 1.0f / l;
     bf16* op = out + (size_t)token * a.out_stride + (size_t)head * HD;
@@ -376,8 +399,13 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(HD <
     const unsigned char* k_base = (const unsigned char*)(kc + (size_t)kvh * (16 * HD));
     const unsigned char* v_base = (const unsigned char*)(vc + (size_t)kvh * (16 * HD));
     size_t page_stride = (size_t)a.n_kv_heads * (16 * HD) * sizeof(bf16);
-    int n = (t_end - t_begin + 31) >> 5;             // tiles of the block, numbered from 0
-    int lp0 = t_begin >> 4;                          // the first tile's first logical page
+    // Tiles of the block, numbered from 0: first those of the kept first keys that lie before the window's tiles (at
+    // most 32 of them; the kept keys among the window's tiles pass the mask there), then the window's.
+    const ScoreBend bend{a.softcap, a.softcap > 0.0f ? a.scale / a.softcap : 0.0f, a.keep_first};
+    int ns = (a.keep_first > 0 && t_begin > 0) ? (min(a.keep_first, t_begin) + 31) >> 5 : 0;
+    int n = ns + ((t_end - t_begin + 31) >> 5);
+    auto tile_t0 = [&](int tile) { return tile < ns ? 32 * tile : t_begin + 32 * (tile - ns); };
+    int lp0 = t_begin >> 4;                          // the first window tile's first logical page
     // The request's page numbers for 64 logical pages at a time, one in each lane.
     int pv_base = lp0;
     auto load_pages = [&](int first) {
@@ -385,13 +413,16 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(HD <
         return min(max(pg, 0), a.num_pages - 1);
     };
     int pv = load_pages(pv_base);
+    int pv_kept = ns > 0 ? load_pages(0) : 0;        // (the pages of the kept keys' tiles)
     // Everything read from memory so far (the queries above all) is waited for here, once: a wait
     // for it inside the loop would be a wait for all of the loop's own loads each time round.
     wait_vmcnt_all();
     auto page_of = [&](int tile) {                   // the page this wave loads from, for a tile in [0, n)
-        int lp = lp0 + 2 * tile;
+        if (tile < ns) return (size_t)__builtin_amdgcn_readlane(pv_kept, 2 * tile + (wave & 1)) * page_stride;
+        int tw = tile - ns;
+        int lp = lp0 + 2 * tw;
         // a tile's second page may lie past the request's last key: then it is not looked up
-        int idx = lp - pv_base + (((wave & 1) && t_begin + 32 * tile + 16 < t_end) ? 1 : 0);
+        int idx = lp - pv_base + (((wave & 1) && t_begin + 32 * tw + 16 < t_end) ? 1 : 0);
         return (size_t)__builtin_amdgcn_readlane(pv, idx) * page_stride;
     };
     auto load_part = [&](const unsigned char* src, const unsigned (&goff)[HALF], int lds_off) {
@@ -408,8 +439,9 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(HD <
     // loaded once more, into a slot that nobody reads; that costs less than telling the cases apart.
     auto issue = [&](int t, int t_mod) {
         int tk = min(t + R, n - 1), tv = min(max(t + R - 1, 0), n - 1);
-        if (__builtin_expect(lp0 + 2 * tk + 1 - pv_base >= 64, 0)) {      // tv <= tk: its pages stay in the window
-            pv_base = lp0 + 2 * tv;
+        int wk = tk - ns, wv = max(tv - ns, 0);                                // their numbers among the window's tiles
+        if (__builtin_expect(wk >= 0 && lp0 + 2 * wk + 1 - pv_base >= 64, 0)) {      // tv <= tk: its pages stay in the window
+            pv_base = lp0 + 2 * wv;
             pv = load_pages(pv_base);
         }
         load_part(k_base + page_of(tk), goff_k, ((t_mod + R) % R) * TILE_BYTES);
@@ -474,7 +506,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(HD <
     };
     // some column of the wave has a key of tile t masked (tiles beyond a wave's own keys are
     // masked as a whole: every wave walks all of the block's tiles)
-    auto is_edge = [&](int t) { int t0 = t_begin + 32 * t; return t0 + 31 > w_first || t0 < w_lo_last; };
+    auto is_edge = [&](int t) { int t0 = tile_t0(t); return t < ns || t0 + 31 > w_first || t0 < w_lo_last; };
     auto to_bf16 = [&](const f32x16& S, bf16x8 (&pf)[2]) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -505,11 +537,11 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(HD <
             if (is_edge(t)) {
                 S_next = scores((s + 1) % R);         // (nothing real for the last tile: not used then)
                 read_values(s, vf);
-                moved = softmax_tile(S_cur, m, l, t_begin + 32 * t, pos, lo, h, scale_log2e, alpha, true, far, far_r1, far_r2);
+                moved = softmax_tile(S_cur, m, l, tile_t0(t), pos, lo, h, scale_log2e, alpha, true, far, far_r1, far_r2, bend);
             } else {
                 S_next = scores((s + 1) % R);
                 read_values(s, vf);
-                moved = softmax_tile(S_cur, m, l, t_begin + 32 * t, pos, lo, h, scale_log2e, alpha, false, far, far_r1, far_r2);
+                moved = softmax_tile(S_cur, m, l, tile_t0(t), pos, lo, h, scale_log2e, alpha, false, far, far_r1, far_r2, bend);
             }
             to_bf16(S_cur, pf);
             rescale(moved, alpha);
@@ -585,9 +617,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 3
 #pragma unroll
         for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
     float m = -INFINITY, l = 0.0f;
+    const ScoreBend bend{a.softcap, a.softcap > 0.0f ? a.scale / a.softcap : 0.0f, a.keep_first};
+    if (!plain && ch == 0 && a.keep_first > 0 && t_begin > 0)          // the first chunk's wave also takes the kept first keys
+        attend_range<HD>(qf, O, m, l, kc, vc, table, a.table_width, a.num_pages,
+                         a.n_kv_heads, kvh, 0, min(a.keep_first, t_begin), pos, lo_t, a.scale, false, 0,
+                         a.dist_r1 != nullptr, a.dist_r1 ? a.dist_r1[head] : 0.0f, a.dist_r1 ? a.dist_r2[head] : 0.0f, bend);
     attend_range<HD>(qf, O, m, l, kc, vc, table, a.table_width, a.num_pages,
                      a.n_kv_heads, kvh, t_begin, t_end, pos, lo_t, a.scale, plain != 0, first_pages,
-                     a.dist_r1 != nullptr, a.dist_r1 ? a.dist_r1[head] : 0.0f, a.dist_r1 ? a.dist_r2[head] : 0.0f);
+                     a.dist_r1 != nullptr, a.dist_r1 ? a.dist_r1[head] : 0.0f, a.dist_r1 ? a.dist_r2[head] : 0.0f, bend);
     if (!cvalid) return;
     float* pp = partial + ((size_t)(e * a.n_heads + head) * max_chunks + ch) * (HD + 2);
     if (h == 0) { pp[0] = m; pp[1] = l; }
@@ -679,7 +716,13 @@ __global__ __launch_bounds__(64) void attn_split16_kernel(const bf16* __restrict
     const bool far = a.dist_r1 != nullptr;
     const float far_r1 = far ? a.dist_r1[head] : 0.0f, far_r2 = far ? a.dist_r2[head] : 0.0f;
     const float c2s = a.scale * 1.44269504088896341f;
-    float c2 = far ? 1.0f : c2s;                      // with the penalty the scores are brought to base 2 before the maximum
+    const ScoreBend bend{a.softcap, a.softcap > 0.0f ? a.scale / a.softcap : 0.0f, a.keep_first};
+    const bool capped = bend.cap > 0.0f;
+    float c2 = (far || capped) ? 1.0f : c2s;          // with the penalty or the cap the scores are brought to base 2 before the maximum
+    // The first chunk's wave also takes the kept first keys that lie before its chunk, in a walk of their own before
+    // the chunk's (those inside the chunk pass the mask there).
+    const int kept_end = (!plain && ch == 0 && a.keep_first > 0 && t_begin > 0) ? min(a.keep_first, t_begin) : 0;
+    const int chunk_begin = t_begin, chunk_end = t_end;
     f32x4 O[HD / 16];
 #pragma unroll
     for (int dt = 0; dt < HD / 16; ++dt) O[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -706,6 +749,13 @@ __global__ __launch_bounds__(64) void attn_split16_kernel(const bf16* __restrict
     };
     bf16x8 kf[2][HD / 32];
     int p0 = 0, p1 = 0;
+    for (int walk = kept_end > 0 ? 0 : 1; walk < 2; ++walk) {
+    if (kept_end > 0) {                                // (the same in all lanes) this walk's keys and their page numbers
+        t_begin = walk == 0 ? 0 : chunk_begin;
+        t_end = walk == 0 ? kept_end : chunk_end;
+        pv_base = t_begin >> 4;
+        pv = load_pages(pv_base);
+    }
     if constexpr (KEYS_AHEAD) {
         pages_of(t_begin, p0, p1);
         load_keys(kf, p0, p1);
@@ -739,18 +789,22 @@ __global__ __launch_bounds__(64) void attn_split16_kernel(const bf16* __restrict
         float sc[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) sc[i] = S[i >> 2][i & 3];
+        if (capped) {                                                 // (the same in all lanes) the soft cap, base 2
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sc[i] = bent_score_log2(sc[i], bend);
+        }
         if (far) {                                                    // (the same in all lanes) the distance penalty, base 2
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 float d = (float)max(pos_t - (t0 + 8 * g + i), 0);
-                sc[i] = __builtin_fmaf(sc[i], c2s, -far_r1 * __builtin_amdgcn_logf(__builtin_fmaf(far_r2, d, 1.0f)));
+                sc[i] = __builtin_fmaf(sc[i], capped ? 1.0f : c2s, -far_r1 * __builtin_amdgcn_logf(__builtin_fmaf(far_r2, d, 1.0f)));
             }
         }
         if (t0 + 31 > pos_t || t0 < lo_t) {                           // (the same in all lanes)
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 int key = t0 + 8 * g + i;
-                if (key > pos_t || key < lo_t) sc[i] = -INFINITY;
+                if (key > pos_t || (key < lo_t && key >= bend.keep)) sc[i] = -INFINITY;
             }
         }
         float mx = sc[0];
@@ -785,6 +839,7 @@ __global__ __launch_bounds__(64) void attn_split16_kernel(const bf16* __restrict
                 p0 = n0; p1 = n1;
             }
         }
+    }
     }
     l = across_groups_sum(l);
     if (!cvalid) return;
@@ -1149,7 +1204,7 @@ int llmrs_attention_bf16_mfma(hipStream_t stream, const bf16* q, bf16* out, cons
     (void)token_entry;
     int G = a.n_heads / a.n_kv_heads;
     if (a.v_dim != a.head_dim) return 0;               // (a distance penalty is these kernels' too)
-    if (a.softcap > 0.0f || a.keep_first > 0) return 0;   // soft-capped scores and kept first keys: the caller's other kernels
+    if (a.keep_first > 1024) return 0;                 // (the tiles of kept first keys: at most 32 a block)
     if (a.page_size != 16 || a.head_dim % 32 || G > 32 || q_starts == nullptr) return 0;
     if (a.q_stride % 8 || a.out_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)out & 7)) return 0;
     if (n_entries > 65535 || a.n_kv_heads > 65535) return 0;

@@ -8,13 +8,12 @@
 // and what stands around them: the activation of q, k and v where a projection leaves them raw, unit norms of q and k
 // with the decay and the write strength of a gated delta rule, the RMS norm of the read-out under a sigmoid gate.
 // Every column of S (one value channel) evolves by itself, so the columns are shared out over lanes; a column's rows
-// are shared out over LANES_PER_COLUMN lanes that add their partial dot products up by cross-lane moves.  A step's
+// are shared out over 8 to 32 lanes that add their partial dot products up by cross-lane moves.  A step's
 // entries (prompt portions and single tokens alike) each start from their request's state and leave it.
 #include "common.h"
 
-#define LANES_PER_COLUMN 8
 #define SCAN_THREADS 256
-#define COLUMNS_PER_BLOCK (SCAN_THREADS / LANES_PER_COLUMN)
+#define SCAN_WAVES (SCAN_THREADS / 64)
 
 struct LinearScanArgs {
     const float* q; int ldq;            // [T, qk_heads * dk]
@@ -28,20 +27,35 @@ struct LinearScanArgs {
     int heads, qk_heads, dk, dv;
 };
 
+template <int P>
 __device__ __forceinline__ float column_sum(float x) {
 #pragma unroll
-    for (int d = 1; d < LANES_PER_COLUMN; d <<= 1) x += __shfl_xor(x, d, 64);
+    for (int d = 1; d < P; d <<= 1) x += __shfl_xor(x, d, 64);
     return x;
 }
 
-// R: rows of a column that one lane holds (rows part * R .. part * R + R - 1; those past dk are idle).
-// VEC: dk % 4 == 0 and all row strides and bases allow 16-byte loads of four consecutive rows.
-template <int R, bool VEC, bool DELTA, bool CHANNEL_DECAY>
+// P lanes share a column, each holding R of its rows (rows part * R .. part * R + R - 1; those past dk are idle: their
+// keys and queries read as zero).  A block is four waves on 4 * 64 / P neighbouring columns of one head and one entry.
+// A token's operands are the same for all of them: the block brings the q, k (and decay) rows of the next CHUNK tokens
+// into LDS, through registers, while it folds the current CHUNK in, so that the walk from token to token waits for LDS
+// and arithmetic only, never for memory.
+template <int P, int R, bool DELTA, bool CHANNEL_DECAY>
 __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(const int* __restrict__ q_starts, const int* __restrict__ slots,
                                                                     LinearScanArgs a) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int part = lane & (LANES_PER_COLUMN - 1);
-    const int col = blockIdx.x * COLUMNS_PER_BLOCK + wave * (64 / LANES_PER_COLUMN) + (lane >> 3);
+    constexpr int DKP = P * R;                              // rows with the idle ones
+    constexpr int CPW = 64 / P, CPB = SCAN_WAVES * CPW;     // columns of a wave, of a block
+    constexpr int CHUNK = 2048 / DKP < 16 ? 2048 / DKP : 16;
+    constexpr int NROW = CHUNK * DKP / SCAN_THREADS;        // elements of an operand's chunk that a thread brings
+    static_assert(R % 4 == 0 && CHUNK >= 1 && CHUNK * DKP % SCAN_THREADS == 0, "rows are read four at a time");
+    __shared__ __attribute__((aligned(16))) float sk[2][CHUNK][DKP];
+    __shared__ __attribute__((aligned(16))) float sq[2][CHUNK][DKP];
+    __shared__ __attribute__((aligned(16))) float sg[CHANNEL_DECAY ? 2 : 1][CHANNEL_DECAY ? CHUNK : 1][CHANNEL_DECAY ? DKP : 4];
+    __shared__ float sv[2][CHUNK][CPB];
+    __shared__ float sb[2][CHUNK];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int part = lane & (P - 1);
+    const int cb = wave * CPW + lane / P;                   // this lane's column within the block
+    const int col = blockIdx.x * CPB + cb;
     const int h = blockIdx.y, e = blockIdx.z;
     const int kh = h / (a.heads / a.qk_heads);
     const bool live = col < a.dv;
@@ -55,75 +69,90 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(const int* __
     for (int i = 0; i < R; ++i) s[i] = (r0 + i < a.dk) ? sp[(size_t)(r0 + i) * a.dv] : 0.0f;
     const float head_decay = (!CHANNEL_DECAY && a.decay) ? a.decay[h] : 1.0f;
 
-    float kc[R], qc[R], gc[CHANNEL_DECAY ? R : 1];
-    float vc = 0.0f, bc = 1.0f;
-    auto fetch = [&](int t, float (&kk)[R], float (&qq)[R], float (&gg)[CHANNEL_DECAY ? R : 1], float& vv, float& bb) {
-        const float* kp = a.k + (size_t)t * a.ldk + (size_t)kh * a.dk + r0;
-        const float* qp = a.q + (size_t)t * a.ldq + (size_t)kh * a.dk + r0;
-        const float* gp = CHANNEL_DECAY ? a.g + (size_t)t * a.ldg + (size_t)h * a.dk + r0 : nullptr;
-        if constexpr (VEC) {
+    // what this thread brings of a chunk: elements tid, tid + 256, ... of [CHUNK][DKP], and one value or write strength
+    constexpr int NV = (CHUNK * CPB + SCAN_THREADS - 1) / SCAN_THREADS;     // values of a chunk that a thread brings
+    float rk[NROW], rq[NROW], rg[CHANNEL_DECAY ? NROW : 1], rv[NV], rb = 1.0f;
+    auto fetch = [&](int tc) {
 #pragma unroll
-            for (int i = 0; i < R; i += 4) {
-                bool in = r0 + i < a.dk;          // (dk % 4 == 0: four rows are in or out together)
-                float4 x = in ? *(const float4*)(kp + i) : make_float4(0, 0, 0, 0);
-                float4 y = in ? *(const float4*)(qp + i) : make_float4(0, 0, 0, 0);
-                kk[i] = x.x; kk[i + 1] = x.y; kk[i + 2] = x.z; kk[i + 3] = x.w;
-                qq[i] = y.x; qq[i + 1] = y.y; qq[i + 2] = y.z; qq[i + 3] = y.w;
+        for (int n = 0; n < NROW; ++n) {
+            int idx = tid + n * SCAN_THREADS, i = idx / DKP, r = idx - i * DKP;
+            int t = tc + i;
+            bool in = t < t1 && r < a.dk;
+            rk[n] = in ? a.k[(size_t)t * a.ldk + (size_t)kh * a.dk + r] : 0.0f;
+            rq[n] = in ? a.q[(size_t)t * a.ldq + (size_t)kh * a.dk + r] : 0.0f;
+            if constexpr (CHANNEL_DECAY) rg[n] = in ? a.g[(size_t)t * a.ldg + (size_t)h * a.dk + r] : 1.0f;
+        }
+#pragma unroll
+        for (int n = 0; n < NV; ++n) {
+            int idx = tid + n * SCAN_THREADS, i = idx / CPB, c = idx - i * CPB, t = tc + i, cc = blockIdx.x * CPB + c;
+            rv[n] = (idx < CHUNK * CPB && t < t1 && cc < a.dv) ? a.v[(size_t)t * a.ldv + (size_t)h * a.dv + cc] : 0.0f;
+        }
+        if (DELTA && tid < CHUNK) rb = tc + tid < t1 ? a.beta[(size_t)(tc + tid) * a.ldb + h] : 0.0f;
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int n = 0; n < NROW; ++n) {
+            int idx = tid + n * SCAN_THREADS, i = idx / DKP, r = idx - i * DKP;
+            sk[buf][i][r] = rk[n];
+            sq[buf][i][r] = rq[n];
+            if constexpr (CHANNEL_DECAY) sg[buf][i][r] = rg[n];
+        }
+#pragma unroll
+        for (int n = 0; n < NV; ++n) {
+            int idx = tid + n * SCAN_THREADS;
+            if (idx < CHUNK * CPB) sv[buf][idx / CPB][idx % CPB] = rv[n];
+        }
+        if (DELTA && tid < CHUNK) sb[buf][tid] = rb;
+    };
+    fetch(t0);
+    stash(0);
+    __syncthreads();
+    int buf = 0;
+    for (int tc = t0; tc < t1; tc += CHUNK, buf ^= 1) {
+        const bool more = tc + CHUNK < t1;
+        if (more) fetch(tc + CHUNK);                    // on its way while this chunk is folded in
+        const int n_here = min(CHUNK, t1 - tc);
+        for (int i = 0; i < n_here; ++i) {
+            float kc[R], qc[R], gc[CHANNEL_DECAY ? R : 1];
+#pragma unroll
+            for (int x = 0; x < R; x += 4) {
+                float4 kk = *(const float4*)&sk[buf][i][r0 + x];
+                float4 qq = *(const float4*)&sq[buf][i][r0 + x];
+                kc[x] = kk.x; kc[x + 1] = kk.y; kc[x + 2] = kk.z; kc[x + 3] = kk.w;
+                qc[x] = qq.x; qc[x + 1] = qq.y; qc[x + 2] = qq.z; qc[x + 3] = qq.w;
                 if constexpr (CHANNEL_DECAY) {
-                    float4 z = in ? *(const float4*)(gp + i) : make_float4(1, 1, 1, 1);
-                    gg[i] = z.x; gg[i + 1] = z.y; gg[i + 2] = z.z; gg[i + 3] = z.w;
+                    float4 gg = *(const float4*)&sg[buf][i][r0 + x];
+                    gc[x] = gg.x; gc[x + 1] = gg.y; gc[x + 2] = gg.z; gc[x + 3] = gg.w;
                 }
             }
-        } else {
+            float u = sv[buf][i][cb];
+            if constexpr (DELTA) {
+                float d0 = 0.0f, d1 = 0.0f;
 #pragma unroll
-            for (int i = 0; i < R; ++i) {
-                bool in = r0 + i < a.dk;
-                kk[i] = in ? kp[i] : 0.0f;
-                qq[i] = in ? qp[i] : 0.0f;
-                if constexpr (CHANNEL_DECAY) gg[i] = in ? gp[i] : 1.0f;
+                for (int x = 0; x < R; x += 2) {
+                    s[x] *= CHANNEL_DECAY ? gc[x] : head_decay;
+                    s[x + 1] *= CHANNEL_DECAY ? gc[x + 1] : head_decay;
+                    d0 = fmaf(kc[x], s[x], d0);
+                    d1 = fmaf(kc[x + 1], s[x + 1], d1);
+                }
+                u = sb[buf][i] * (u - column_sum<P>(d0 + d1));
+            } else {
+#pragma unroll
+                for (int x = 0; x < R; ++x) s[x] *= CHANNEL_DECAY ? gc[x] : head_decay;
             }
-        }
-        vv = a.v[(size_t)t * a.ldv + (size_t)h * a.dv + j];
-        bb = DELTA ? a.beta[(size_t)t * a.ldb + h] : 1.0f;
-    };
-    fetch(t0, kc, qc, gc, vc, bc);
-    for (int t = t0; t < t1; ++t) {
-        float kn[R], qn[R], gn[CHANNEL_DECAY ? R : 1];
-        float vn = 0.0f, bn = 1.0f;
-        if (t + 1 < t1) fetch(t + 1, kn, qn, gn, vn, bn);          // the next token's operands travel while this one is folded in
-        float u = vc;
-        if constexpr (DELTA) {
-            float d0 = 0.0f, d1 = 0.0f;
+            float o0 = 0.0f, o1 = 0.0f;
 #pragma unroll
-            for (int i = 0; i < R; i += 2) {
-                s[i] *= CHANNEL_DECAY ? gc[i] : head_decay;
-                s[i + 1] *= CHANNEL_DECAY ? gc[i + 1] : head_decay;
-                d0 = fmaf(kc[i], s[i], d0);
-                d1 = fmaf(kc[i + 1], s[i + 1], d1);
+            for (int x = 0; x < R; x += 2) {
+                s[x] = fmaf(kc[x], u, s[x]);
+                s[x + 1] = fmaf(kc[x + 1], u, s[x + 1]);
+                o0 = fmaf(qc[x], s[x], o0);
+                o1 = fmaf(qc[x + 1], s[x + 1], o1);
             }
-            u = bc * (vc - column_sum(d0 + d1));
-        } else {
-#pragma unroll
-            for (int i = 0; i < R; ++i) s[i] *= CHANNEL_DECAY ? gc[i] : head_decay;
+            float o = column_sum<P>(o0 + o1);
+            if (live && part == 0) a.out[(size_t)(tc + i) * a.ldo + (size_t)h * a.dv + j] = o;
         }
-        float o0 = 0.0f, o1 = 0.0f;
-#pragma unroll
-        for (int i = 0; i < R; i += 2) {
-            s[i] = fmaf(kc[i], u, s[i]);
-            s[i + 1] = fmaf(kc[i + 1], u, s[i + 1]);
-            o0 = fmaf(qc[i], s[i], o0);
-            o1 = fmaf(qc[i + 1], s[i + 1], o1);
-        }
-        float o = column_sum(o0 + o1);
-        if (live && part == 0) a.out[(size_t)t * a.ldo + (size_t)h * a.dv + j] = o;
-        if (t + 1 < t1) {
-#pragma unroll
-            for (int i = 0; i < R; ++i) {
-                kc[i] = kn[i]; qc[i] = qn[i];
-                if constexpr (CHANNEL_DECAY) gc[i] = gn[i];
-            }
-            vc = vn; bc = bn;
-        }
+        if (more) stash(buf ^ 1);                       // (the other buffer: nobody reads it during this chunk)
+        __syncthreads();
     }
     if (live) {
 #pragma unroll
@@ -142,7 +171,7 @@ extern "C" int llmrs_linear_scan(hipStream_t stream, const float* q, int ldq, co
                                  long state_stride, const int* q_starts, const int* slots, int n_entries, int n_tokens,
                                  int heads, int qk_heads, int dk, int dv, float* out, int ldo) {
     LLMRS_REQUIRE(heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && dk > 0 && dv > 0, "linear_scan: bad sizes");
-    LLMRS_REQUIRE(dk <= 32 * LANES_PER_COLUMN, "linear_scan: %d key channels exceed %d", dk, 32 * LANES_PER_COLUMN);
+    LLMRS_REQUIRE(dk <= 512, "linear_scan: %d key channels exceed 512", dk);
     LLMRS_REQUIRE(ldq >= qk_heads * dk && ldk >= qk_heads * dk && ldv >= heads * dv && ldo >= heads * dv, "linear_scan: row stride too short");
     LLMRS_REQUIRE(!g || ldg >= heads * dk, "linear_scan: the decays' rows are too short");
     LLMRS_REQUIRE(!(g && decay), "linear_scan: a decay per head or per channel, not both");
@@ -151,17 +180,12 @@ extern "C" int llmrs_linear_scan(hipStream_t stream, const float* q, int ldq, co
     LLMRS_REQUIRE(entries_given(q_starts, slots, n_entries), "linear_scan: bad entries");
     if (n_tokens == 0) return 0;
     LinearScanArgs a{q, ldq, k, ldk, v, ldv, g, ldg, decay, beta, ldb, state, state_stride, out, ldo, heads, qk_heads, dk, dv};
-    int per_lane = ceil_div(dk, LANES_PER_COLUMN);
-    int R = per_lane <= 4 ? 4 : per_lane <= 8 ? 8 : per_lane <= 16 ? 16 : 32;
-    auto aligned = [](const void* p, int ld) { return ((uintptr_t)p & 15) == 0 && ld % 4 == 0; };
-    bool vec = dk % 4 == 0 && aligned(q, ldq) && aligned(k, ldk) && (!g || aligned(g, ldg));
-    dim3 grid(ceil_div(dv, COLUMNS_PER_BLOCK), heads, n_entries);
-#define SCAN(RR, V, D, C) linear_scan_kernel<RR, V, D, C><<<grid, SCAN_THREADS, 0, stream>>>(q_starts, slots, a)
-#define BY_ROWS(V, D, C) do { if (R == 4) SCAN(4, V, D, C); else if (R == 8) SCAN(8, V, D, C); else if (R == 16) SCAN(16, V, D, C); else SCAN(32, V, D, C); } while (0)
-#define BY_KIND(V) do { if (beta && g) BY_ROWS(V, true, true); else if (beta) BY_ROWS(V, true, false); else if (g) BY_ROWS(V, false, true); else BY_ROWS(V, false, false); } while (0)
-    if (vec) BY_KIND(true); else BY_KIND(false);
-#undef BY_KIND
-#undef BY_ROWS
+    // lanes to a column and rows to a lane by the number of key channels: eight rows a lane where that fills the lanes
+#define SCAN(PP, RR, D, C) linear_scan_kernel<PP, RR, D, C><<<dim3(ceil_div(dv, SCAN_WAVES * 64 / PP), heads, n_entries), SCAN_THREADS, 0, stream>>>(q_starts, slots, a)
+#define BY_SIZE(D, C) do { if (dk <= 32) SCAN(8, 4, D, C); else if (dk <= 64) SCAN(8, 8, D, C); else if (dk <= 128) SCAN(16, 8, D, C); \
+                           else if (dk <= 256) SCAN(32, 8, D, C); else SCAN(32, 16, D, C); } while (0)
+    if (beta && g) BY_SIZE(true, true); else if (beta) BY_SIZE(true, false); else if (g) BY_SIZE(false, true); else BY_SIZE(false, false);
+#undef BY_SIZE
 #undef SCAN
     LLMRS_LAUNCH_CHECK("linear_scan");
     return 0;

@@ -104,3 +104,87 @@ extern "C" int llmrs_act_weight(hipStream_t stream, int dtype, const float* up, 
     LLMRS_LAUNCH_CHECK("act_weight");
     return 0;
 }
+
+// ---- the experts' rows one after the other --------------------------------------------------------------------------
+// For steps of many tokens the chosen (token, expert) pairs are laid out expert by expert, each expert's rows in the
+// order of their tokens, so that an expert's tokens are a dense product of their own.  counts[e]: how many tokens chose
+// expert e (a wave an expert).  With the counts known: row_token[row], row_weight[row] for every row, and
+// row_of[t, e] = the row of token t with expert e, or -1 (a wave an expert; an expert's first row is the sum of the
+// counts before it).
+__global__ __launch_bounds__(64) void route_counts_kernel(const float* __restrict__ weights, int ldw, int T, int* __restrict__ counts) {
+    int e = blockIdx.x, lane = threadIdx.x, n = 0;
+    for (int t = lane; t < T; t += 64) n += weights[(size_t)t * ldw + e] > 0.0f;
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) n += __shfl_xor(n, d, 64);
+    if (lane == 0) counts[e] = n;
+}
+
+__global__ __launch_bounds__(64) void route_rows_kernel(const float* __restrict__ weights, int ldw, int T, int E, const int* __restrict__ counts,
+                                                         int* __restrict__ row_token, float* __restrict__ row_weight, int* __restrict__ row_of) {
+    int e = blockIdx.x, lane = threadIdx.x, first = 0;
+    for (int i = lane; i < e; i += 64) first += counts[i];
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) first += __shfl_xor(first, d, 64);
+    for (int t0 = 0; t0 < T; t0 += 64) {
+        int t = t0 + lane;
+        float w = t < T ? weights[(size_t)t * ldw + e] : 0.0f;
+        unsigned long long chosen = __ballot(w > 0.0f);
+        int row = first + __popcll(chosen & ((1ull << lane) - 1ull));
+        if (t < T) row_of[(size_t)t * E + e] = w > 0.0f ? row : -1;
+        if (w > 0.0f) { row_token[row] = t; row_weight[row] = w; }
+        first += __popcll(chosen);
+    }
+}
+
+extern "C" int llmrs_route_counts(hipStream_t stream, const float* weights, int ldw, int n_tokens, int E, int* counts) {
+    LLMRS_REQUIRE(weights && counts && E > 0 && ldw >= E && n_tokens >= 0 && E <= 65535, "route_counts: bad arguments");
+    route_counts_kernel<<<E, 64, 0, stream>>>(weights, ldw, n_tokens, counts);
+    LLMRS_LAUNCH_CHECK("route_counts");
+    return 0;
+}
+
+extern "C" int llmrs_route_rows(hipStream_t stream, const float* weights, int ldw, int n_tokens, int E, const int* counts, int* row_token,
+                                float* row_weight, int* row_of) {
+    LLMRS_REQUIRE(weights && counts && row_token && row_weight && row_of && E > 0 && ldw >= E && n_tokens >= 0 && E <= 65535, "route_rows: bad arguments");
+    route_rows_kernel<<<E, 64, 0, stream>>>(weights, ldw, n_tokens, E, counts, row_token, row_weight, row_of);
+    LLMRS_LAUNCH_CHECK("route_rows");
+    return 0;
+}
+
+// out[r, :] = x[rows[r], :] (rows of the activation type)
+template <class T>
+__global__ void gather_rows_kernel(T* __restrict__ out, int ldo, const T* __restrict__ x, int ldx, const int* __restrict__ rows, int D) {
+    int r = blockIdx.x, src = rows[r];
+    for (int d = threadIdx.x; d < D; d += blockDim.x) out[(size_t)r * ldo + d] = x[(size_t)src * ldx + d];
+}
+
+extern "C" int llmrs_gather_rows(hipStream_t stream, int dtype, void* out, int ldo, const void* x, int ldx, const int* rows, int n_rows, int D) {
+    LLMRS_REQUIRE(out && x && rows && D > 0 && ldo >= D && ldx >= D && n_rows >= 0, "gather_rows: bad arguments");
+    if (n_rows == 0) return 0;
+    if (dtype == LLMRS_F32) gather_rows_kernel<float><<<n_rows, 256, 0, stream>>>((float*)out, ldo, (const float*)x, ldx, rows, D);
+    else if (dtype == LLMRS_BF16) gather_rows_kernel<bf16><<<n_rows, 256, 0, stream>>>((bf16*)out, ldo, (const bf16*)x, ldx, rows, D);
+    else return llmrs_fail("gather_rows: unknown dtype %d", dtype);
+    LLMRS_LAUNCH_CHECK("gather_rows");
+    return 0;
+}
+
+// h[t, :] += sum over the experts e that token t chose, in ascending e, of y[row_of[t, e], :]; 32-bit.
+__global__ void combine_rows_kernel(float* __restrict__ h, int ldh, const float* __restrict__ y, int ldy, const int* __restrict__ row_of, int E, int D) {
+    int t = blockIdx.x;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float acc = 0.0f;
+        for (int e = 0; e < E; ++e) {
+            int row = row_of[(size_t)t * E + e];
+            if (row >= 0) acc += y[(size_t)row * ldy + d];
+        }
+        h[(size_t)t * ldh + d] += acc;
+    }
+}
+
+extern "C" int llmrs_combine_rows(hipStream_t stream, float* h, int ldh, const float* y, int ldy, const int* row_of, int n_tokens, int E, int D) {
+    LLMRS_REQUIRE(h && y && row_of && D > 0 && ldh >= D && ldy >= D && E > 0 && n_tokens >= 0, "combine_rows: bad arguments");
+    if (n_tokens == 0) return 0;
+    combine_rows_kernel<<<n_tokens, 256, 0, stream>>>(h, ldh, y, ldy, row_of, E, D);
+    LLMRS_LAUNCH_CHECK("combine_rows");
+    return 0;
+}

@@ -201,6 +201,10 @@ class HipKernels(Kernels):
             "llmrs_route_topk": [V, V, I, V, I, I, I, I, I],
             "llmrs_act_weight": [V, I, V, I, V, I, I, I, I, I, V, I],
             "llmrs_add_bias_rows": [V, V, I, V, I, I],
+            "llmrs_route_counts": [V, V, I, I, I, V],
+            "llmrs_route_rows": [V, V, I, I, I, V, V, V, V],
+            "llmrs_gather_rows": [V, I, V, I, V, I, V, I, I],
+            "llmrs_combine_rows": [V, V, I, V, I, V, I, I, I],
             "llmrs_mingru_scan": [V, I, V, I, V, V, V, ctypes.c_long, V, V, I, I, V, I, I, V],
             "llmrs_causal_conv_silu": [V, I, V, I, V, V, V, ctypes.c_long, V, V, V, I, I, I, I, V, I],
             "llmrs_selective_scan": [V, I, V, I, V, I, I, I, V, I, V, V, V, V, I, V, ctypes.c_long, V, V, V, I, I, I, I, V, I, I, V],
@@ -611,6 +615,33 @@ class HipKernels(Kernels):
         T, E = logits.shape
         self._run(f"route_topk {T}x{E}", T * E * 8, 8 * T * E, None, self.lib.llmrs_route_topk, self._stream(), _p(logits),
                   logits.stride(0), _p(weights), weights.stride(0), T, E, int(top), int(bool(renormalize)))
+
+    def route_counts(self, weights: torch.Tensor, counts: torch.Tensor) -> None:
+        """counts[e] = how many tokens chose expert e (weights[t, e] > 0); weights float32 [T, E], counts int32 [E]."""
+        assert weights.dtype == torch.float32 and weights.stride(1) == 1 and counts.dtype == torch.int32 and counts.numel() == weights.shape[1]
+        self._run("route_counts", weights.numel() * 4, 0, None, self.lib.llmrs_route_counts, self._stream(), _p(weights), weights.stride(0),
+                  weights.shape[0], weights.shape[1], _p(counts))
+
+    def route_rows(self, weights: torch.Tensor, counts: torch.Tensor, row_token: torch.Tensor, row_weight: torch.Tensor, row_of: torch.Tensor) -> None:
+        """The chosen (token, expert) pairs expert by expert, each expert's in the order of their tokens: row_token and
+        row_weight [rows], row_of [T, E] (the pair's row, or -1)."""
+        T, E = weights.shape
+        assert row_token.dtype == row_of.dtype == torch.int32 and row_weight.dtype == torch.float32 and row_of.is_contiguous() and tuple(row_of.shape) == (T, E)
+        self._run("route_rows", weights.numel() * 8, 0, None, self.lib.llmrs_route_rows, self._stream(), _p(weights), weights.stride(0), T, E,
+                  _p(counts), _p(row_token), _p(row_weight), _p(row_of))
+
+    def gather_rows(self, out: torch.Tensor, x: torch.Tensor, rows: torch.Tensor) -> None:
+        """out[r] = x[rows[r]]; rows int32."""
+        assert out.dtype == x.dtype and out.stride(1) == x.stride(1) == 1 and out.shape[1] == x.shape[1] and rows.dtype == torch.int32 and rows.numel() == out.shape[0]
+        self._run(f"gather_rows {out.shape[0]}x{out.shape[1]}", 2 * out.numel() * out.element_size(), 0, None, self.lib.llmrs_gather_rows,
+                  self._stream(), _code(out.dtype), _p(out), out.stride(0), _p(x), x.stride(0), _p(rows), out.shape[0], out.shape[1])
+
+    def combine_rows(self, h: torch.Tensor, y: torch.Tensor, row_of: torch.Tensor) -> None:
+        """h[t] += the sum of y[row_of[t, e]] over the experts e with row_of[t, e] >= 0, in ascending e; float32."""
+        assert h.dtype == y.dtype == torch.float32 and h.stride(1) == y.stride(1) == 1 and h.shape[1] == y.shape[1]
+        assert row_of.dtype == torch.int32 and row_of.is_contiguous() and row_of.shape[0] == h.shape[0]
+        self._run(f"combine_rows {h.shape[0]}x{h.shape[1]}", (y.numel() + 2 * h.numel()) * 4, y.numel(), None, self.lib.llmrs_combine_rows,
+                  self._stream(), _p(h), h.stride(0), _p(y), y.stride(0), _p(row_of), h.shape[0], row_of.shape[1], h.shape[1])
 
     def act_weight(self, out: torch.Tensor, up: torch.Tensor, weights: Optional[torch.Tensor], ff: int) -> None:
         """out[t, c] = relu(up[t, c])^2 * (weights[t, c // ff] if weights is given); up, weights float32."""

@@ -105,8 +105,13 @@ class RoutedFF(FeedForward):
     The experts' up matrices are laid one under the other and their down matrices side by side at load, so a step's
     experts are one up product of experts * intermediate_size columns, one pass that applies the activation and each
     column's expert weight (zero where the token did not choose the expert), and one down product: w_e Wdown_e act(.)
-    = Wdown_e (w_e act(.)).  Names: `router`, and `expert` with a place for the expert's number (e.g. "e{}")."""
+    = Wdown_e (w_e act(.)).  A step with a prompt portion (never one that is recorded) whose experts would each get
+    `SORT_FROM_ROWS` rows or more on average lays the chosen (token, expert) pairs out expert by expert instead, and
+    every expert's rows are a product of their own: top / experts of the arithmetic.  The host reads how many tokens
+    each expert got (one small copy) to size those products; the down matrices are kept a second time, one by one.
+    Names: `router`, and `expert` with a place for the expert's number (e.g. "e{}")."""
     graph_safe = True
+    SORT_FROM_ROWS = 128
 
     def __init__(self, spec, dtype):
         super().__init__(spec, dtype)
@@ -123,7 +128,7 @@ class RoutedFF(FeedForward):
         self.n_router = self.name(leaves["router"])
         self.n_up = [self.name(leaves["expert"].format(e) + "." + leaves["up"]) for e in range(self.experts)]
         self.n_down = [self.name(leaves["expert"].format(e) + "." + leaves["down"]) for e in range(self.experts)]
-        self.w_router = self.w_up = self.w_down = None
+        self.w_router = self.w_up = self.w_down = self.w_down_each = None
 
     def tensors(self):
         t = {self.n_router: TensorSpec((self.experts, self.hidden), "normal:0.0:0.1")}
@@ -136,6 +141,9 @@ class RoutedFF(FeedForward):
         self.w_router = place(tensors[self.n_router], device, self.dtype)
         self.w_up = torch.cat([place(tensors[n], device, self.dtype) for n in self.n_up], dim=0).contiguous()
         self.w_down = torch.cat([place(tensors[n], device, self.dtype) for n in self.n_down], dim=1).contiguous()
+        # each expert's down matrix by itself, for the steps that run the experts one by one (not when all are chosen)
+        self.w_down_each = (self.w_down.view(self.hidden, self.experts, self.inter).permute(1, 0, 2).contiguous()
+                            if self.top < self.experts else None)
 
     def export(self):
         up, down = self.w_up.cpu(), self.w_down.cpu()
@@ -147,6 +155,8 @@ class RoutedFF(FeedForward):
 
     def step_weight_bytes(self, seen):
         # a single token reads the router and the experts it chose
+        if self.w_down_each is not None:
+            seen.add(self.w_down_each.data_ptr())          # (the second copy of the down matrices: a step reads one of the two)
         total = super().step_weight_bytes(seen)
         experts = (self.w_up.numel() + self.w_down.numel()) * self.w_up.element_size()
         return total - experts + experts * self.top // self.experts
@@ -158,11 +168,50 @@ class RoutedFF(FeedForward):
         k.gemm(x, self.w_router, logits, EPI_STORE_F32, ctx.gemm_workspace(x, self.w_router))
         weights = ctx.workspace("moe.weights", (T, self.experts), torch.float32)
         k.route_topk(logits, weights, self.top, self.renormalize)
+        if self.w_down_each is not None and ctx.longest > 1 and T * self.top >= self.SORT_FROM_ROWS * self.experts:
+            return self._forward_sorted(ctx, x, h, weights)
         up = ctx.workspace("mlp.up", (T, N), torch.float32)
         k.gemm(x, self.w_up, up, EPI_STORE_F32, ctx.gemm_workspace(x, self.w_up))
         act = ctx.workspace("mlp.act", (T, N), self.dtype)
         k.act_weight(act, up, weights, self.inter)
         k.gemm(act, self.w_down, h, EPI_ACCUM_F32, ctx.gemm_workspace(act, self.w_down))
+        ctx.note_left(h, None)
+
+
+    def _forward_sorted(self, ctx, x, h, weights):
+        k = kernels()
+        T, E, F, D = x.shape[0], self.experts, self.inter, self.hidden
+        rows = T * self.top
+        counts = ctx.workspace("moe.counts", (E,), torch.int32)
+        k.route_counts(weights, counts)
+        n_of = counts.cpu().tolist()                 # (the step waits here: the experts' products are sized by these)
+        total = sum(n_of)                            # (a chosen expert whose score is exactly zero has no row: it adds nothing)
+        assert total <= rows
+        row_token = ctx.workspace("moe.row_token", (rows,), torch.int32)
+        row_weight = ctx.workspace("moe.row_weight", (rows, 1), torch.float32)
+        row_of = ctx.workspace("moe.row_of", (T, E), torch.int32)
+        k.route_rows(weights, counts, row_token, row_weight, row_of)
+        if total == 0:
+            return ctx.note_left(h, None)
+        xs = ctx.workspace("moe.x", (rows, D), self.dtype)[:total]
+        k.gather_rows(xs, x, row_token[:total])
+        up = ctx.workspace("mlp.up", (rows, F), torch.float32)[:total]
+        at = 0
+        for e, n in enumerate(n_of):
+            if n:
+                w = self.w_up[e * F:(e + 1) * F]
+                k.gemm(xs[at:at + n], w, up[at:at + n], EPI_STORE_F32, ctx.gemm_workspace(xs[at:at + n], w))
+                at += n
+        act = ctx.workspace("mlp.act", (rows, F), self.dtype)[:total]
+        k.act_weight(act, up, row_weight[:total], F)
+        ys = ctx.workspace("moe.y", (rows, D), torch.float32)[:total]
+        at = 0
+        for e, n in enumerate(n_of):
+            if n:
+                w = self.w_down_each[e]
+                k.gemm(act[at:at + n], w, ys[at:at + n], EPI_STORE_F32, ctx.gemm_workspace(act[at:at + n], w))
+                at += n
+        k.combine_rows(h, ys, row_of)
         ctx.note_left(h, None)
 
 

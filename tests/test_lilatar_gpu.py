@@ -232,6 +232,30 @@ def test_experts_of_which_some_are_chosen(experts, top, dtype):
                 {"whole": whole(requests), "decoded": tail_decoded(requests, tail=5), "portions": portions(requests, (2, 3))})
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("experts,top", [(4, 1), (5, 2), (16, 4)])
+def test_experts_run_one_by_one_over_their_own_tokens(experts, top, dtype, monkeypatch):
+    """Steps with prompt portions lay the chosen (token, expert) pairs out expert by expert (here from the first row on,
+    not only for long steps); single decoded tokens beside them keep to the product over all experts."""
+    from llm_rs_amd.parts import RoutedFF
+    monkeypatch.setattr(RoutedFF, "SORT_FROM_ROWS", 0)
+    cfg = one_layer(lightning(2, 8, 8, mlp=moe(10, experts, top)), width=48)
+    typed, tensors = make_model(cfg, seed=experts)
+    need = 1e-4 if dtype == "float32" else 0.03
+    found = []
+    for seed in range(2000):
+        toks = random_tokens(cfg["vocab"], 8 if dtype == "bfloat16" else 70, seed)
+        if routed_layer_margin(cfg, tensors, toks) > need:
+            found.append(toks)
+            if len(found) == 3:
+                break
+    assert len(found) == 3, "no sequences with clear choices found"
+    requests = {f"r{i}": t for i, t in enumerate(found)}
+    run_regimes(cfg, typed, tensors, dtype, 4, requests,
+                {"whole": whole(requests), "decoded": tail_decoded(requests, tail=5), "portions": portions(requests, (2, 3, 30)),
+                 "mixed": mixed(requests, live=3, prefill_sizes=(3, 2, 9))})
+
+
 # ---- whole models in every regime -----------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", DTYPES)
