@@ -636,6 +636,10 @@ def run_lilatar(args) -> dict:
     """Prompt and decode throughput of the Lilatar decoder at two widths, each beside a Llama decoder of the same
     width, heads, feed-forward and number of layers (random weights both)."""
     repeats = max(1, (args.layers or 6) // 3)
+    if args.experts_by_rows_from is not None:
+        from llm_rs_amd.parts import RoutedFF
+        RoutedFF.SORT_FROM_ROWS = args.experts_by_rows_from
+        RoutedFF.SORT_FROM_WEIGHT = 0
     sizes = {"1B widths": (LLAMA_1B, 2048, 32, 8, 64, 8192), "8B widths": (LLAMA_8B, 4096, 32, 8, 128, 14336)}
     pairs = {size: {"lilatar": lilatar_shape(width, heads, kv_heads, dim, ff, args.window, repeats, args.experts, args.top),
                     "llama": dict(llama, num_hidden_layers=3 * repeats)}
@@ -672,6 +676,8 @@ def main() -> int:
     ap.add_argument("--only-size", default="", help="tuvodra, lilatar: run one of the sizes only (1B or 8B)")
     ap.add_argument("--experts", type=int, default=16, help="lilatar: experts of a routed feed-forward")
     ap.add_argument("--top", type=int, default=4, help="lilatar: experts a token uses")
+    ap.add_argument("--experts-by-rows-from", type=int, default=None,
+                    help="lilatar: rows an expert gets on average from which a prompt step runs the experts one by one (default: the part's own rule)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")

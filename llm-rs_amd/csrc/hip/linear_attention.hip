@@ -27,10 +27,27 @@ struct LinearScanArgs {
     int heads, qk_heads, dk, dv;
 };
 
+// The sum of a value over the P neighbouring lanes that share a column, left in all of them.  The moves between lanes
+// are the vector unit's own (quads, half rows and rows of 16 lanes mirrored; for 32 lanes the register swap between
+// neighbouring rows of 16): a few cycles each, where a move through the LDS crossbar costs a trip there, and a token's
+// two sums stand in the chain from token to token.
+template <int CTRL>
+__device__ __forceinline__ float lanes_moved(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float neighbouring_row(float x) {
+    unsigned u = __float_as_uint(x);
+    auto sw = __builtin_amdgcn_permlane16_swap(u, u, false, false);      // {rows 0, 0, 2, 2 of x; rows 1, 1, 3, 3 of x}
+    return __uint_as_float((threadIdx.x & 16) ? sw[0] : sw[1]);
+}
 template <int P>
 __device__ __forceinline__ float column_sum(float x) {
-#pragma unroll
-    for (int d = 1; d < P; d <<= 1) x += __shfl_xor(x, d, 64);
+    static_assert(P == 8 || P == 16 || P == 32, "8, 16 or 32 lanes to a column");
+    x += lanes_moved<0xB1>(x);                   // quad_perm [1, 0, 3, 2]: the neighbour
+    x += lanes_moved<0x4E>(x);                   // quad_perm [2, 3, 0, 1]: the other pair of the quad
+    x += lanes_moved<0x141>(x);                  // row_half_mirror: the other quad of the eight
+    if constexpr (P >= 16) x += lanes_moved<0x140>(x);       // row_mirror: the other eight of the sixteen
+    if constexpr (P >= 32) x += neighbouring_row(x);
     return x;
 }
 

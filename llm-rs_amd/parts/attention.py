@@ -85,6 +85,9 @@ class Attention(Mixer):
         self.w_qkv = None
         self.w_o = None
         self.bias = self.o_bias = self.r1 = self.r2 = None
+        # Set by a part that holds this mixer and adds the output projection's bias itself, in a pass over the output
+        # that it makes anyway (it reads the bias from `o_bias`): `forward` then leaves the bias out.
+        self.output_bias_left_to_holder = False
 
     def tensors(self):
         n = self.names
@@ -183,7 +186,7 @@ class Attention(Mixer):
                     scratch, ctx.max_seq_len, ctx.n_single, self._keys_for_the_split(ctx), value_dim=self.value_dim,
                     distance=None if self.distance is None else (self.r1, self.r2), softcap=self.softcap, keep_first=self.keep_first)
         k.gemm(o, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(o, self.w_o))
-        if self.has_o_bias:
+        if self.has_o_bias and not self.output_bias_left_to_holder:
             k.add_bias_rows(h, self.o_bias)
         ctx.note_left(h, None)
 
@@ -258,7 +261,7 @@ class Attention(Mixer):
                     self._keys_for_the_split(ctx))
         leave = ctx.room_for_next_norm(h, self.w_o) if not self.has_o_bias else None
         k.gemm(o, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(o, self.w_o), **({} if leave is None else {"leave": leave}))
-        if self.has_o_bias:
+        if self.has_o_bias and not self.output_bias_left_to_holder:
             k.add_bias_rows(h, self.o_bias)
         ctx.note_left(h, leave)
 

@@ -67,9 +67,6 @@ class Lightning(Mixer):
         return {n["q"]: w[:a].contiguous(), n["k"]: w[a:b].contiguous(), n["v"]: w[b:c].contiguous(), n["gate"]: w[c:].contiguous(),
                 n["out"]: self.w_o.cpu(), n["norm"]: self.norm.cpu()}
 
-    def step_weight_bytes(self, seen):
-        return super().step_weight_bytes(seen)
-
     def cache_need(self):
         return FixedState((self.heads * self.dk * self.dv,), torch.float32)
 
@@ -193,7 +190,7 @@ class Parallel(Mixer):
         keyed = [m for m, _ in self.branches if m.recording_signature is not None]
         self._keyed = keyed
         self.recording_signature = tuple(m.recording_signature for m in keyed) or None
-        self.out_weights = []
+        self.out_weights, self.out_biases = [], []
         # the branches' needs, in their order; a branch without a need has no part in the view
         self._needs = [m.cache_need() for m, _ in self.branches]
 
@@ -208,10 +205,15 @@ class Parallel(Mixer):
         return t
 
     def load(self, tensors, device):
-        self.out_weights = []
+        self.out_weights, self.out_biases = [], []
         for m, out in self.branches:
             m.load(tensors, device)
             self.out_weights.append(place(tensors[out], device, torch.float32))
+            # a branch whose output projection has a bias leaves it to the kernel that norms the branches' outputs
+            bias = getattr(m, "o_bias", None) if hasattr(m, "output_bias_left_to_holder") else None
+            if bias is not None:
+                m.output_bias_left_to_holder = True
+            self.out_biases.append(bias)
 
     def export(self):
         t = {}
@@ -235,7 +237,7 @@ class Parallel(Mixer):
         views = iter(cache.parts)
         for i, (m, _) in enumerate(self.branches):
             m.forward(ctx, x, ys[i], next(views) if self._needs[i] is not None else None)
-        k.rmsnorm_sum(h, [(ys[i], None, w) for i, w in enumerate(self.out_weights)], 1.0 / len(self.branches), self.eps)
+        k.rmsnorm_sum(h, [(ys[i], b, w) for i, (w, b) in enumerate(zip(self.out_weights, self.out_biases))], 1.0 / len(self.branches), self.eps)
         ctx.note_left(h, None)
 
 

@@ -239,6 +239,7 @@ def test_experts_run_one_by_one_over_their_own_tokens(experts, top, dtype, monke
     not only for long steps); single decoded tokens beside them keep to the product over all experts."""
     from llm_rs_amd.parts import RoutedFF
     monkeypatch.setattr(RoutedFF, "SORT_FROM_ROWS", 0)
+    monkeypatch.setattr(RoutedFF, "SORT_FROM_WEIGHT", 0)
     cfg = one_layer(lightning(2, 8, 8, mlp=moe(10, experts, top)), width=48)
     typed, tensors = make_model(cfg, seed=experts)
     need = 1e-4 if dtype == "float32" else 0.03
