@@ -22,7 +22,8 @@ struct LinearScanArgs {
     const float* g; int ldg;            // [T, heads * dk] decay per key channel, or null
     const float* decay;                 // [heads] decay per head, or null (both null: none)
     const float* beta; int ldb;         // [T, heads] write strength of the delta rule, or null: plain linear attention
-    float* state; long state_stride;    // [slots][heads][dk][dv]
+    float* state; long state_stride;    // [slots][heads][dv][dk]: a column's rows side by side, as a lane reads and leaves them
+    int state_vec;                      // rows of the state may be read four at a time (dk % 4 == 0, 16-byte aligned slots)
     float* out; int ldo;                // [T, heads * dv]
     int heads, qk_heads, dk, dv;
 };
@@ -80,10 +81,18 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(const int* __
     const int r0 = part * R;
     const int t0 = q_starts[e], t1 = q_starts[e + 1];
     if (t0 >= t1) return;
-    float* sp = a.state + (size_t)slots[e] * a.state_stride + (size_t)h * a.dk * a.dv + j;
+    float* sp = a.state + (size_t)slots[e] * a.state_stride + ((size_t)h * a.dv + j) * a.dk + r0;
     float s[R];
+    if (a.state_vec) {
 #pragma unroll
-    for (int i = 0; i < R; ++i) s[i] = (r0 + i < a.dk) ? sp[(size_t)(r0 + i) * a.dv] : 0.0f;
+        for (int i = 0; i < R; i += 4) {
+            float4 x = r0 + i < a.dk ? *(const float4*)(sp + i) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            s[i] = x.x; s[i + 1] = x.y; s[i + 2] = x.z; s[i + 3] = x.w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < R; ++i) s[i] = (r0 + i < a.dk) ? sp[i] : 0.0f;
+    }
     const float head_decay = (!CHANNEL_DECAY && a.decay) ? a.decay[h] : 1.0f;
 
     // what this thread brings of a chunk: elements tid, tid + 256, ... of [CHUNK][DKP], and one value or write strength
@@ -172,16 +181,22 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(const int* __
         __syncthreads();
     }
     if (live) {
+        if (a.state_vec) {
 #pragma unroll
-        for (int i = 0; i < R; ++i)
-            if (r0 + i < a.dk) sp[(size_t)(r0 + i) * a.dv] = s[i];
+            for (int i = 0; i < R; i += 4)
+                if (r0 + i < a.dk) *(float4*)(sp + i) = make_float4(s[i], s[i + 1], s[i + 2], s[i + 3]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+                if (r0 + i < a.dk) sp[i] = s[i];
+        }
     }
 }
 
 static bool entries_given(const int* q_starts, const int* slots, int n_entries) { return q_starts && slots && n_entries > 0 && n_entries <= 65535; }
 
 // q, k: [T, qk_heads * dk]; v: [T, heads * dv]; g: [T, heads * dk] or null; decay: [heads] or null; beta: [T, heads] or
-// null (no delta correction); state: [slots][heads * dk * dv] at state_stride floats a slot, read at an entry's first
+// null (no delta correction); state: [slots][heads][dv][dk] at state_stride floats a slot, read at an entry's first
 // token and left at its last; out: [T, heads * dv].  All 32-bit.  Head h reads the q and k of head h / (heads / qk_heads).
 extern "C" int llmrs_linear_scan(hipStream_t stream, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv,
                                  const float* g, int ldg, const float* decay, const float* beta, int ldb, float* state,
@@ -196,7 +211,8 @@ extern "C" int llmrs_linear_scan(hipStream_t stream, const float* q, int ldq, co
     LLMRS_REQUIRE(state_stride >= (long)heads * dk * dv && heads <= 65535, "linear_scan: the state does not fit its slot");
     LLMRS_REQUIRE(entries_given(q_starts, slots, n_entries), "linear_scan: bad entries");
     if (n_tokens == 0) return 0;
-    LinearScanArgs a{q, ldq, k, ldk, v, ldv, g, ldg, decay, beta, ldb, state, state_stride, out, ldo, heads, qk_heads, dk, dv};
+    int state_vec = dk % 4 == 0 && state_stride % 4 == 0 && ((uintptr_t)state & 15) == 0;
+    LinearScanArgs a{q, ldq, k, ldk, v, ldv, g, ldg, decay, beta, ldb, state, state_stride, state_vec, out, ldo, heads, qk_heads, dk, dv};
     // lanes to a column and rows to a lane by the number of key channels: eight rows a lane where that fills the lanes
 #define SCAN(PP, RR, D, C) linear_scan_kernel<PP, RR, D, C><<<dim3(ceil_div(dv, SCAN_WAVES * 64 / PP), heads, n_entries), SCAN_THREADS, 0, stream>>>(q_starts, slots, a)
 #define BY_SIZE(D, C) do { if (dk <= 32) SCAN(8, 4, D, C); else if (dk <= 64) SCAN(8, 8, D, C); else if (dk <= 128) SCAN(16, 8, D, C); \

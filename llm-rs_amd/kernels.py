@@ -547,7 +547,8 @@ class HipKernels(Kernels):
         """Per head a matrix S [dk, dv] carried from token to token: S <- decay S (decay [heads], or g [T, heads * dk] a
         key channel); u = beta (v - S^T k) (beta [T, heads]; None: u = v); S <- S + k u^T; out = S^T q.  q, k
         [T, qk_heads * dk], v and out [T, heads * dv], all float32 with unit column stride; state [slots, >= heads * dk * dv]
-        float32, read at an entry's first token and left at its last."""
+        float32, laid out [heads][dv][dk] (a value channel's key channels side by side), read at an entry's first token
+        and left at its last."""
         T = q.shape[0]
         for t in (q, k, v, out, g, beta):
             assert t is None or (t.dtype == torch.float32 and t.stride(1) == 1 and t.shape[0] == T)

@@ -200,7 +200,7 @@ class EmulatedKernels(Kernels):
     def linear_scan(self, q, k, v, state, q_starts, slots, heads, qk_heads, dk, dv, out, decay=None, g=None, beta=None):
         rep = heads // qk_heads
         for e in range(slots.numel()):
-            S = state[int(slots[e])][:heads * dk * dv].view(heads, dk, dv)
+            S = state[int(slots[e])][:heads * dk * dv].view(heads, dv, dk).transpose(1, 2)       # kept value channel by key channel
             for t in range(int(q_starts[e]), int(q_starts[e + 1])):
                 qt = q[t].view(qk_heads, dk).repeat_interleave(rep, dim=0)
                 kt = k[t].view(qk_heads, dk).repeat_interleave(rep, dim=0)
