@@ -50,6 +50,15 @@ class LilatarConfig:
         self.logit_scale = float(d.get("logit_scale", 1.0))
         self.eps = float(_need(_need(d, "norm", ""), "eps", "norm."))
         self.layers: List[Dict[str, Any]] = copy.deepcopy(list(_need(d, "layers", "")))
+        for layer in self.layers:           # what a file may leave out: as many key heads as heads; one decay for all heads
+            m = layer.get("mixer") if isinstance(layer, dict) else None
+            if not isinstance(m, dict):
+                continue
+            for side in (m.get("left"), m.get("right")):
+                if isinstance(side, dict) and side.get("kv_heads") is None and side.get("heads") is not None:
+                    side["kv_heads"] = side["heads"]
+            if isinstance(m.get("decay"), (int, float)) and m.get("heads") is not None:
+                m["decay"] = [float(m["decay"])] * int(m["heads"])
         self.validate()
 
     @classmethod

@@ -38,6 +38,20 @@ def test_a_missing_key_is_named(path):
         LilatarConfig.from_dict(d).model_spec()
 
 
+def test_what_a_file_may_leave_out():
+    d = copy.deepcopy(CONFIGS["plain"])
+    del d["layers"][1]["mixer"]["right"]["kv_heads"], d["layers"][2]["mixer"]["left"]["kv_heads"], d["logit_scale"]
+    d["layers"][0]["mixer"]["decay"] = 0.9
+    d["layers"][1]["mixer"]["left"]["softcap"] = None
+    cfg = LilatarConfig.from_dict(d)
+    spec = cfg.model_spec()
+    assert spec.logit_scale == 1.0 and spec.layers[0].mixer.params["decay"] == [0.9] * 4
+    branches = spec.layers[1].mixer.params["branches"]
+    assert branches[1]["mixer"].params["kv_heads"] == 4 and branches[0]["mixer"].params["softcap"] == 0.0
+    assert spec.layers[2].mixer.params["branches"][0]["mixer"].params["num_kv_heads"] == 2
+    assert cfg.to_dict()["layers"][0]["mixer"]["decay"] == [0.9] * 4
+
+
 def test_what_does_not_fit_is_refused():
     for change in (lambda d: d["layers"][0].update(type="attention"), lambda d: d["layers"][0]["mixer"]["left"].update(kv_heads=4),
                    lambda d: d["layers"][1]["mlp"].update(kind="gated"), lambda d: d["layers"][1]["mixer"].update(decay=[0.5]),

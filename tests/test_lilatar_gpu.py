@@ -324,7 +324,10 @@ def shows(cfg, tensors, toks, at, where):
 
 # head shapes: values narrower than keys (the kernel for any sizes) and heads the matrix-core kernels take
 HEAD_SHAPES = {"any sizes": dict(dim=16, vdim=12, heads=2, kv_heads=1, width=32, rot_dims=8),
-               "matrix cores": dict(dim=64, vdim=64, heads=4, kv_heads=2, width=64, rot_dims=32)}
+               "matrix cores": dict(dim=64, vdim=64, heads=4, kv_heads=2, width=64, rot_dims=32),
+               "matrix cores, heads of 128": dict(dim=128, vdim=128, heads=2, kv_heads=1, width=64, rot_dims=64),
+               "matrix cores, heads of 32 in threes": dict(dim=32, vdim=32, heads=3, kv_heads=1, width=64, rot_dims=16),
+               "matrix cores, twenty heads to a key head": dict(dim=32, vdim=32, heads=20, kv_heads=1, width=64, rot_dims=32)}
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -338,7 +341,7 @@ def test_a_key_just_inside_and_just_outside_the_window(window, at, shape, dtype)
     exact = reference(cfg, tensors, requests)
     inside, outside = at + window - 1, at + window
     seen, unseen = shows(cfg, tensors, toks, at, inside), shows(cfg, tensors, toks, at, outside)
-    assert seen > 0.05 and unseen < 1e-9, (seen, unseen)
+    assert seen > 0.03 and unseen < 1e-9, (seen, unseen)
     allowed = allowed_error(dtype, cfg, tensors, requests, exact)
     assert allowed < seen / 2, (allowed, seen)
     regimes = {"whole": whole(requests), "decoded over the edge": tail_decoded(requests, tail=8),
@@ -362,9 +365,9 @@ def test_the_last_kept_token_and_the_first_that_is_not(keep, window, shape, dtyp
         requests = {"m": toks}
         exact = reference(cfg, tensors, requests)
         late = shows(cfg, tensors, toks, at, n - 1)
-        assert (late > 0.05) if stays else (late < 1e-9), (at, late)
+        assert (late > 0.03) if stays else (late < 1e-9), (at, late)
         allowed = allowed_error(dtype, cfg, tensors, requests, exact)
-        assert allowed < 0.2            # (less than half of what the marked token moves where it is seen)
+        assert allowed < (late / 2 if stays else 0.2), (allowed, late)      # (less than half of what the marked token moves where it is seen)
         for name, steps in {"whole": whole(requests), "decoded": tail_decoded(requests, tail=40), "portions": portions(requests, (64, 3, 130, 2)),
                             "portions of two": portions(requests, (2,)) if keep == 4 else None}.items():
             if steps is None:
