@@ -334,6 +334,9 @@ extern "C" int llmrs_gated_rmsnorm(hipStream_t stream, int dtype, const float* x
 // ---- sums of normed rows added into the stream ---------------------------------------------------------------------
 // out[t, :] += coef * sum_i rmsnorm(x_i[t, :] + bias_i) * w_i,   i < n_in (1 or 2), all 32-bit, rows of D.
 // The norm after a sublayer (n_in = 1, coef = 1), and the mean of two mixers' normed outputs (n_in = 2, coef = 1/2).
+// HELD > 0: rows of up to 256 * HELD columns, which a thread keeps in registers between the two passes (everything a
+// row needs from memory is then asked for at once); HELD == 0: any length, the rows read twice.
+template <int HELD>
 __global__ __launch_bounds__(256) void rmsnorm_sum_kernel(float* __restrict__ out, const float* __restrict__ x0, const float* __restrict__ b0,
                                                            const float* __restrict__ w0, const float* __restrict__ x1,
                                                            const float* __restrict__ b1, const float* __restrict__ w1, int D,
@@ -342,13 +345,31 @@ __global__ __launch_bounds__(256) void rmsnorm_sum_kernel(float* __restrict__ ou
     int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* r0 = x0 + (size_t)t * D;
     const float* r1 = x1 ? x1 + (size_t)t * D : nullptr;
+    float* orow = out + (size_t)t * D;
+    constexpr int N = HELD > 0 ? HELD : 1;
+    float a[N], b[N], wa[N], wb[N], o[N];
     float s0 = 0.0f, s1 = 0.0f;
-    for (int d = threadIdx.x; d < D; d += 256) {
-        float a = r0[d] + (b0 ? b0[d] : 0.0f);
-        s0 = fmaf(a, a, s0);
-        if (r1) {
-            float b = r1[d] + (b1 ? b1[d] : 0.0f);
-            s1 = fmaf(b, b, s1);
+    if constexpr (HELD > 0) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            int d = threadIdx.x + 256 * i;
+            bool in = d < D;
+            a[i] = in ? r0[d] + (b0 ? b0[d] : 0.0f) : 0.0f;
+            b[i] = in && r1 ? r1[d] + (b1 ? b1[d] : 0.0f) : 0.0f;
+            wa[i] = in ? w0[d] : 0.0f;
+            wb[i] = in && r1 ? w1[d] : 0.0f;
+            o[i] = in ? orow[d] : 0.0f;
+            s0 = fmaf(a[i], a[i], s0);
+            s1 = fmaf(b[i], b[i], s1);
+        }
+    } else {
+        for (int d = threadIdx.x; d < D; d += 256) {
+            float u = r0[d] + (b0 ? b0[d] : 0.0f);
+            s0 = fmaf(u, u, s0);
+            if (r1) {
+                float v = r1[d] + (b1 ? b1[d] : 0.0f);
+                s1 = fmaf(v, v, s1);
+            }
         }
     }
     s0 = wave_sum(s0);
@@ -357,11 +378,20 @@ __global__ __launch_bounds__(256) void rmsnorm_sum_kernel(float* __restrict__ ou
     __syncthreads();
     float inv0 = 1.0f / sqrtf((partial[0][0] + partial[0][1] + partial[0][2] + partial[0][3]) / (float)D + eps);
     float inv1 = 1.0f / sqrtf((partial[1][0] + partial[1][1] + partial[1][2] + partial[1][3]) / (float)D + eps);
-    float* orow = out + (size_t)t * D;
-    for (int d = threadIdx.x; d < D; d += 256) {
-        float y = (r0[d] + (b0 ? b0[d] : 0.0f)) * inv0 * w0[d];
-        if (r1) y += (r1[d] + (b1 ? b1[d] : 0.0f)) * inv1 * w1[d];
-        orow[d] += coef * y;
+    if constexpr (HELD > 0) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            int d = threadIdx.x + 256 * i;
+            float y = a[i] * inv0 * wa[i];
+            if (r1) y += b[i] * inv1 * wb[i];
+            if (d < D) orow[d] = o[i] + coef * y;
+        }
+    } else {
+        for (int d = threadIdx.x; d < D; d += 256) {
+            float y = (r0[d] + (b0 ? b0[d] : 0.0f)) * inv0 * w0[d];
+            if (r1) y += (r1[d] + (b1 ? b1[d] : 0.0f)) * inv1 * w1[d];
+            orow[d] += coef * y;
+        }
     }
 }
 
@@ -370,7 +400,9 @@ extern "C" int llmrs_rmsnorm_sum(hipStream_t stream, float* out, const float* x0
     LLMRS_REQUIRE(out && x0 && w0 && D > 0 && n_rows >= 0, "rmsnorm_sum: bad arguments");
     LLMRS_REQUIRE((x1 == nullptr) == (w1 == nullptr) && (x1 || !b1), "rmsnorm_sum: the second input needs rows and a weight");
     if (n_rows == 0) return 0;
-    rmsnorm_sum_kernel<<<n_rows, 256, 0, stream>>>(out, x0, b0, w0, x1, b1, w1, D, coef, eps);
+    if (D <= 256 * 4) rmsnorm_sum_kernel<4><<<n_rows, 256, 0, stream>>>(out, x0, b0, w0, x1, b1, w1, D, coef, eps);
+    else if (D <= 256 * 16) rmsnorm_sum_kernel<16><<<n_rows, 256, 0, stream>>>(out, x0, b0, w0, x1, b1, w1, D, coef, eps);
+    else rmsnorm_sum_kernel<0><<<n_rows, 256, 0, stream>>>(out, x0, b0, w0, x1, b1, w1, D, coef, eps);
     LLMRS_LAUNCH_CHECK("rmsnorm_sum");
     return 0;
 }
