@@ -400,8 +400,10 @@ extern "C" int llmrs_rmsnorm_sum(hipStream_t stream, float* out, const float* x0
     LLMRS_REQUIRE(out && x0 && w0 && D > 0 && n_rows >= 0, "rmsnorm_sum: bad arguments");
     LLMRS_REQUIRE((x1 == nullptr) == (w1 == nullptr) && (x1 || !b1), "rmsnorm_sum: the second input needs rows and a weight");
     if (n_rows == 0) return 0;
-    if (D <= 256 * 4) rmsnorm_sum_kernel<4><<<n_rows, 256, 0, stream>>>(out, x0, b0, w0, x1, b1, w1, D, coef, eps);
-    else if (D <= 256 * 16) rmsnorm_sum_kernel<16><<<n_rows, 256, 0, stream>>>(out, x0, b0, w0, x1, b1, w1, D, coef, eps);
+    // few rows: one trip to memory for everything a row needs (8 rows of 2048: 5.3 against 7.1 us); many rows: the
+    // second read comes from the cache and more waves fit a unit (2048 rows of 2048: 18 against 21 us)
+    if (n_rows < 256 && D <= 256 * 4) rmsnorm_sum_kernel<4><<<n_rows, 256, 0, stream>>>(out, x0, b0, w0, x1, b1, w1, D, coef, eps);
+    else if (n_rows < 256 && D <= 256 * 16) rmsnorm_sum_kernel<16><<<n_rows, 256, 0, stream>>>(out, x0, b0, w0, x1, b1, w1, D, coef, eps);
     else rmsnorm_sum_kernel<0><<<n_rows, 256, 0, stream>>>(out, x0, b0, w0, x1, b1, w1, D, coef, eps);
     LLMRS_LAUNCH_CHECK("rmsnorm_sum");
     return 0;

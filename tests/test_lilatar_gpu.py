@@ -130,7 +130,7 @@ def test_the_small_kernels_around_the_recurrences(dtype):
         k.gated_rmsnorm(got, x.cuda(), gate.cuda(), w.cuda(), group, 1e-5)
         assert float((got.cpu().float() - want).abs().max()) <= (1e-5 if dtype == torch.float32 else 1e-2) * float(want.abs().max())
     # sums of normed rows into the stream, one and two inputs, with and without a bias
-    for D in (7, 64, 1000, 1030, 4100):
+    for D, T in ((7, 21), (64, 21), (1000, 21), (1030, 21), (4100, 21), (72, 300)):       # (few rows and many: two ways through the rows)
         for n_in in (1, 2):
             ins = [(torch.randn(T, D, generator=g), torch.randn(D, generator=g) if i == 0 and D != 64 else None, torch.randn(D, generator=g)) for i in range(n_in)]
             base = torch.randn(T, D, generator=g)
