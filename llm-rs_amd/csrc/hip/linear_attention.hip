@@ -138,6 +138,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(const int* __
         const bool more = tc + CHUNK < t1;
         if (more) fetch(tc + CHUNK);                    // on its way while this chunk is folded in
         const int n_here = min(CHUNK, t1 - tc);
+#pragma unroll 4
         for (int i = 0; i < n_here; ++i) {
             float kc[R], qc[R], gc[CHANNEL_DECAY ? R : 1];
 #pragma unroll
